@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
     T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink, int chunk_blocks,
-    const float* __restrict__ distance_bias, int bias_span) {
+    const float* __restrict__ distance_bias, int bias_span, int stretch) {
     __shared__ float qs[G * OWNED * XRT_WAVE];                 // [G][head_dim]
     __shared__ float ps[WAVES][G * XRT_WAVE];
     // what the wavefronts found in the chunks of a round, for the merge: two sets, used in turn (WAVES > 1)
@@ -212,7 +212,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
         return;
     }
     const int pos = positions[token];
-    const int first = window > 0 ? max(0, pos - window + 1) : 0;
+    // the first key the query sees: the window's, and with stretches of positions the first of the query's own stretch
+    const int first = max(window > 0 ? max(0, pos - window + 1) : 0, stretch > 0 ? pos - pos % stretch : 0);
     const bool biased = distance_slopes != nullptr;
     float slopes[G];
 #pragma unroll
@@ -302,7 +303,7 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
                           int window, const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
-                          hipStream_t s) {
+                          int stretch, hipStream_t s) {
     XRT_REQUIRE(distance_bias == nullptr || bias_span > 0, "attention: a table of biases by distance needs a distance at least");
     XRT_REQUIRE(head_dim <= MAX_HEAD_DIM && value_dim > 0 && value_dim <= MAX_HEAD_DIM, "attention: head sizes %d and %d must be at most %d", head_dim, value_dim, MAX_HEAD_DIM);
     // Query heads of a key/value head that a wavefront takes together: as many of the group as 4, for head sizes up to 128
@@ -318,12 +319,13 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
     const int row_width = q_stride > 0 ? (int)q_stride : (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim;
     // few (token, head) pairs (a decode step): a workgroup of wavefronts each, which take the chunks of keys side by side
     const bool side_by_side = (long)tokens * n_heads <= 8L * XRT_COMPUTE_UNITS;
-    const int chunk_blocks = window > 0 && window <= WINDOW_FOR_SHORT_CHUNKS ? 1 : CHUNK_BLOCKS;
+    const int sees_at_most = window > 0 && stretch > 0 ? min(window, stretch) : max(window, stretch);     // (0: everything)
+    const int chunk_blocks = sees_at_most > 0 && sees_at_most <= WINDOW_FOR_SHORT_CHUNKS ? 1 : CHUNK_BLOCKS;
     const size_t round_bytes = (size_t)2 * CHUNK_WAVES * together * value_dim * sizeof(float);
 #define XRT_GENERIC(T, WAVES_, G_, OWNED_)                                                                                \
     attention_generic_kernel<T, WAVES_, G_, OWNED_><<<(unsigned)items, WAVES_ * XRT_WAVE, WAVES_ > 1 ? round_bytes : 0, s>>>( \
         (const T*)qkv, row_width, n_heads, n_kv_heads, head_dim, value_dim, (const T*)k_cache, (const T*)v_cache, block_table,       \
-        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, chunk_blocks, distance_bias, bias_span)
+        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, chunk_blocks, distance_bias, bias_span, stretch)
 #define XRT_GENERIC_WAVES(T, G_, OWNED_) do { if (side_by_side) XRT_GENERIC(T, CHUNK_WAVES, G_, OWNED_); else XRT_GENERIC(T, 1, G_, OWNED_); } while (0)
 #define XRT_GENERIC_SETS(T)                                                                                               \
     do {                                                                                                                  \

@@ -43,11 +43,12 @@ __device__ __forceinline__ float conv_input(const T* __restrict__ x, long x_stri
 
 // grid (sequences, segments, channel chunks). phase 0: outputs only; 1: outputs and the state (one segment per sequence);
 // 2: the state only (a launch of its own after phase 0, so that no workgroup reads a state another one is writing).
-template <typename T>
+// bias [n_out][channels] of the filters' type (or null) is added to the sum, then the activation (XRT_CONV_ACT_*) is applied.
+template <typename TI, typename T>
 __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
-    const T* __restrict__ x, long x_stride, int channels, const void* __restrict__ w, int w_dtype, int taps, int n_out, int mode,
+    const TI* __restrict__ x, long x_stride, int channels, const void* __restrict__ w, int w_dtype, int taps, int n_out, int mode,
     float* __restrict__ state, const int* __restrict__ seq_offsets, const int* __restrict__ seq_slots, T* __restrict__ out,
-    long tokens, int phase) {
+    long tokens, int phase, const void* __restrict__ bias, int activation) {
 #pragma clang fp contract(off)      // (only the products and sums written as fmaf are fused: the same in every kernel that does this convolution)
     const int seq = blockIdx.x, c = blockIdx.z * CONV_THREADS + threadIdx.x;
     if (c >= channels) return;
@@ -89,6 +90,8 @@ __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
                 y = fmaf(load_as_float(w, w_dtype, w_at + taps - 1), now, y);
                 if (mode == XRT_CONV_PLUS_INPUT) y += now;
             }
+            if (bias != nullptr) y += load_as_float(bias, w_dtype, (long)o * channels + c);
+            if (activation == XRT_CONV_ACT_SILU) y = silu_exact(y);
             out[((long)o * tokens + begin + t) * channels + c] = from_float<T>(y);
         }
 #pragma unroll
@@ -154,6 +157,17 @@ struct TokenInputs {
     float q[M], k[M], d[M], v;
 };
 
+// XRT_DECAY_STEP: the token's step size of a head, softplus(z + bias), from decay [tokens][decay_stride] and decay_bias [heads]
+__device__ __forceinline__ float step_of(const xrt_recurrence& a, long row, int head) {
+    float z = a.decay[row * a.decay_stride + head];
+    if (a.decay_bias != nullptr) z += load_as_float(a.decay_bias, a.decay_bias_dtype, head);
+    return softplus_exact(z);
+}
+// the head of q and k that `head` reads: heads may share them in groups of neighbours
+__device__ __forceinline__ int qk_head_of(const xrt_recurrence& a, int head) {
+    return a.qk_heads > 0 && a.qk_heads < a.heads ? head / (a.heads / a.qk_heads) : head;
+}
+
 // The decay of key channel `at` (head * dim + channel) at the token in `row`.
 __device__ __forceinline__ float decay_of(const xrt_recurrence& a, long row, int head, long at) {
     if (a.decay_mode == XRT_DECAY_PER_HEAD) return a.decay[head];
@@ -169,18 +183,25 @@ template <int M>
 __device__ __forceinline__ void load_token(TokenInputs<M>& in, const xrt_recurrence& a, int dtype, long row, int head, int column, bool owner,
                                            int row0, int rows) {
     const int lane = threadIdx.x;
+    const bool stepped = a.decay_mode == XRT_DECAY_STEP;
+    float step = 1.f, stepped_decay = 1.f;
+    if (stepped) {                                         // one decay for the head's channels, and the step also scales what is fed
+        step = step_of(a, row, head);
+        stepped_decay = expf(-expf(load_as_float(a.decay_rate, a.decay_rate_dtype, head)) * step);
+    }
+    const int qk_head = qk_head_of(a, head);
 #pragma unroll
     for (int m = 0; m < M; ++m) {
         const int i = lane + XRT_WAVE * m;
         in.q[m] = 0.f; in.k[m] = 0.f; in.d[m] = 1.f;
         if (i < rows) {
-            const long at = (long)head * a.dim + row0 + i;
-            in.q[m] = load_as_float(a.q, dtype, row * a.q_stride + at) * a.q_scale;
-            in.k[m] = load_as_float(a.k, dtype, row * a.k_stride + at) * a.k_scale;
-            in.d[m] = decay_of(a, row, head, at);
+            const long at = (long)head * a.dim + row0 + i, qk_at = (long)qk_head * a.dim + row0 + i;
+            in.q[m] = load_as_float(a.q, dtype, row * a.q_stride + qk_at) * a.q_scale;
+            in.k[m] = load_as_float(a.k, dtype, row * a.k_stride + qk_at) * a.k_scale;
+            in.d[m] = stepped ? stepped_decay : decay_of(a, row, head, at);
         }
     }
-    in.v = owner ? load_as_float(a.v, dtype, row * a.v_stride + (long)head * a.vdim + column) : 0.f;
+    in.v = owner ? load_as_float(a.v, dtype, row * a.v_stride + (long)head * a.vdim + column) * step : 0.f;
 }
 
 // grid (sequences, heads * vslices * row_split, segments), one wavefront each. With row_split > 1 (one segment only) a wavefront
@@ -339,8 +360,8 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_r
     float bonus_dot = 0.f;
     if (a.bonus != nullptr) {
         for (int i = lane; i < a.dim; i += XRT_WAVE) {
-            const long at = (long)head * a.dim + i;
-            const float k = load_as_float(a.k, dtype, row * a.k_stride + at) * a.k_scale, q = load_as_float(a.q, dtype, row * a.q_stride + at) * a.q_scale;
+            const long at = (long)head * a.dim + i, qk_at = (long)qk_head_of(a, head) * a.dim + i;
+            const float k = load_as_float(a.k, dtype, row * a.k_stride + qk_at) * a.k_scale, q = load_as_float(a.q, dtype, row * a.q_stride + qk_at) * a.q_scale;
             bonus_dot = fmaf(load_as_float(a.bonus, a.bonus_dtype, at) * k, q, bonus_dot);
         }
         bonus_dot = wave_sum(bonus_dot);
@@ -350,6 +371,7 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_r
         float sum = raw[out_at + c];
         for (int part = 1; part < row_split; ++part) sum += raw[(long)part * tokens * a.heads * vdim + out_at + c];
         if (a.bonus != nullptr) sum = fmaf(bonus_dot, load_as_float(a.v, dtype, row * a.v_stride + (long)head * vdim + c), sum);
+        if (a.skip != nullptr) sum = fmaf(load_as_float(a.skip, a.skip_dtype, head), load_as_float(a.v, dtype, row * a.v_stride + (long)head * vdim + c), sum);
         return sum;
     };
     float inv = 1.f;
@@ -363,10 +385,43 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_r
         if (a.norm_weight != nullptr)
             value *= load_as_float(a.norm_weight, a.norm_weight_dtype, a.norm_weight_per_head ? (long)head * vdim + c : c);
         if (a.gate != nullptr) {
-            const float g = load_as_float(a.gate, dtype, row * a.gate_stride + (long)head * vdim + c);
+            const float g = load_as_float(a.gate, a.gate_is_float32 ? XRT_F32 : dtype, row * a.gate_stride + (long)head * vdim + c);
             value *= a.gate_act == XRT_GATE_SILU ? silu_exact(g) : g;
         }
         store_from_float(a.out, dtype, out_at + c, value);
+    }
+}
+
+// The same for a norm that comes after the gate and spans equal parts of the token's whole row (heads x vdim), whatever the
+// heads are: value = raw (+ skip * v) times the gate, then divided by the root mean square of its part, times the weight
+// [heads * vdim]. A workgroup per (token, part).
+__global__ void __launch_bounds__(256) recurrence_finish_groups_kernel(const xrt_recurrence a, int dtype, const float* __restrict__ raw,
+                                                                      const int* __restrict__ token_slots, int row_split, long tokens) {
+    __shared__ float scratch[32];
+    const long row = blockIdx.x;
+    const int width = a.heads * a.vdim, part_width = width / a.norm_groups, c0 = blockIdx.y * part_width;
+    const long out_at = row * width;
+    if (token_slots[row] < 0) {
+        for (int c = threadIdx.x; c < part_width; c += blockDim.x) store_from_float(a.out, dtype, out_at + c0 + c, 0.f);
+        return;
+    }
+    auto gated = [&](int c) {                              // c: a column of the whole row
+        float sum = raw[out_at + c];
+        for (int part = 1; part < row_split; ++part) sum += raw[(long)part * tokens * width + out_at + c];
+        if (a.skip != nullptr) sum = fmaf(load_as_float(a.skip, a.skip_dtype, c / a.vdim), load_as_float(a.v, dtype, row * a.v_stride + c), sum);
+        if (a.gate != nullptr) {
+            const float g = load_as_float(a.gate, a.gate_is_float32 ? XRT_F32 : dtype, row * a.gate_stride + c);
+            sum *= a.gate_act == XRT_GATE_SILU ? silu_exact(g) : g;
+        }
+        return sum;
+    };
+    float squares = 0.f;
+    for (int c = threadIdx.x; c < part_width; c += blockDim.x) { const float o = gated(c0 + c); squares = fmaf(o, o, squares); }
+    const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)part_width + a.eps);
+    for (int c = threadIdx.x; c < part_width; c += blockDim.x) {
+        float value = gated(c0 + c) * inv;
+        if (a.norm_weight != nullptr) value *= load_as_float(a.norm_weight, a.norm_weight_dtype, c0 + c);
+        store_from_float(a.out, dtype, out_at + c0 + c, value);
     }
 }
 
@@ -443,33 +498,49 @@ __global__ void kv_store_kernel(const T* __restrict__ k, long k_stride, const T*
 
 }  // namespace
 
-extern "C" int xrt_short_conv(const void* x, int dtype, long tokens, long x_stride, int channels, const void* w, int w_dtype, int taps,
-                              int n_out, int mode, float* state, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
-                              void* out, void* stream) {
+extern "C" int xrt_short_conv_with(const void* x, int dtype, long tokens, long x_stride, int channels, const void* w, int w_dtype, int taps,
+                                   int n_out, int mode, float* state, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
+                                   void* out, int out_dtype, const void* bias, int activation, void* stream) {
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "short_conv: unknown dtype %d", dtype);
+    XRT_REQUIRE(out_dtype == dtype || (dtype == XRT_F32 && out_dtype == XRT_BF16), "short_conv: the result has the input's type, or is bfloat16 of float32 inputs");
     XRT_REQUIRE(w_dtype == XRT_F32 || w_dtype == XRT_BF16, "short_conv: unknown weight dtype %d", w_dtype);
     XRT_REQUIRE(x && w && (state || taps == 1) && seq_offsets && seq_slots && out, "short_conv: null operand");
     XRT_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps, 1 to %d are served", taps, CONV_MAX_TAPS);
     XRT_REQUIRE(mode == XRT_CONV_PLAIN || mode == XRT_CONV_PLUS_INPUT || (mode == XRT_CONV_TOWARDS_LAST && taps == 2),
                 "short_conv: unknown mode %d (the interpolation towards the input before has two taps)", mode);
+    XRT_REQUIRE(activation == XRT_CONV_ACT_NONE || activation == XRT_CONV_ACT_SILU, "short_conv: unknown activation %d", activation);
     XRT_REQUIRE(channels > 0 && n_out > 0 && x_stride >= channels && tokens >= 0 && n_seqs >= 0 && max_count >= 0, "short_conv: bad sizes");
     if (n_seqs == 0 || max_count == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const int segments = (max_count + CONV_SEGMENT - 1) / CONV_SEGMENT;
     const int chunks = (channels + CONV_THREADS - 1) / CONV_THREADS;
     XRT_REQUIRE(segments <= 65535 && chunks <= 65535, "short_conv: a step this long is not served");
-#define XRT_CONV(T, segments_, phase_)                                                                                     \
-    short_conv_kernel<T><<<dim3(n_seqs, segments_, chunks), CONV_THREADS, 0, s>>>((const T*)x, x_stride, channels, w, w_dtype, taps, \
-        n_out, mode, state, seq_offsets, seq_slots, (T*)out, tokens, phase_)
+#define XRT_CONV(TI, T, segments_, phase_)                                                                                     \
+    short_conv_kernel<TI, T><<<dim3(n_seqs, segments_, chunks), CONV_THREADS, 0, s>>>((const TI*)x, x_stride, channels, w, w_dtype, taps, \
+        n_out, mode, state, seq_offsets, seq_slots, (T*)out, tokens, phase_, bias, activation)
+#define XRT_CONV_TYPES(segments_, phase_)                                                          \
+    do {                                                                                           \
+        if (dtype == XRT_F32 && out_dtype == XRT_F32) XRT_CONV(float, float, segments_, phase_);   \
+        else if (dtype == XRT_F32) XRT_CONV(float, bf16, segments_, phase_);                       \
+        else XRT_CONV(bf16, bf16, segments_, phase_);                                              \
+    } while (0)
     if (segments == 1 || taps == 1) {                      // (one tap: no state, nothing that one workgroup writes and another reads)
-        if (dtype == XRT_F32) XRT_CONV(float, segments, 1); else XRT_CONV(bf16, segments, 1);
+        XRT_CONV_TYPES(segments, 1);
     } else {
-        if (dtype == XRT_F32) XRT_CONV(float, segments, 0); else XRT_CONV(bf16, segments, 0);
-        if (dtype == XRT_F32) XRT_CONV(float, 1, 2); else XRT_CONV(bf16, 1, 2);
+        XRT_CONV_TYPES(segments, 0);
+        XRT_CONV_TYPES(1, 2);
     }
+#undef XRT_CONV_TYPES
 #undef XRT_CONV
     XRT_LAUNCH_CHECK("short_conv");
     return 0;
+}
+
+extern "C" int xrt_short_conv(const void* x, int dtype, long tokens, long x_stride, int channels, const void* w, int w_dtype, int taps,
+                              int n_out, int mode, float* state, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
+                              void* out, void* stream) {
+    return xrt_short_conv_with(x, dtype, tokens, x_stride, channels, w, w_dtype, taps, n_out, mode, state, seq_offsets, seq_slots, n_seqs,
+                               max_count, out, dtype, nullptr, XRT_CONV_ACT_NONE, stream);
 }
 
 extern "C" long xrt_linear_recurrence_workspace(int n_seqs, int max_count, long tokens, int heads, int dim, int vdim) {
@@ -487,9 +558,16 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
     XRT_REQUIRE(a.q && a.k && a.v && a.state && a.out, "linear_recurrence: null operand");
     XRT_REQUIRE(a.heads > 0 && a.dim > 0 && a.dim <= 256 && a.vdim > 0 && (long)a.heads * ((a.vdim + XRT_WAVE - 1) / XRT_WAVE) <= 65535,
                 "linear_recurrence: %d heads of %d x %d: key sizes up to 256 are served", a.heads, a.dim, a.vdim);
-    XRT_REQUIRE(a.decay_mode >= XRT_DECAY_PER_HEAD && a.decay_mode <= XRT_DECAY_SIGMOID_POWER && a.decay != nullptr,
+    XRT_REQUIRE(a.decay_mode >= XRT_DECAY_PER_HEAD && a.decay_mode <= XRT_DECAY_STEP && a.decay != nullptr,
                 "linear_recurrence: unknown decay mode %d, or no decays", a.decay_mode);
-    XRT_REQUIRE(a.q_stride >= a.heads * a.dim && a.k_stride >= a.heads * a.dim && a.v_stride >= a.heads * a.vdim &&
+    XRT_REQUIRE(a.decay_mode != XRT_DECAY_STEP || (a.decay_rate != nullptr && a.decay_stride >= a.heads),
+                "linear_recurrence: decays from step sizes need a rate per head and the steps' row stride");
+    XRT_REQUIRE(a.qk_heads == 0 || (a.qk_heads > 0 && a.heads % a.qk_heads == 0), "linear_recurrence: %d heads cannot share %d heads of q and k", a.heads, a.qk_heads);
+    XRT_REQUIRE(a.norm_groups == 0 || (a.norm != 0 && a.norm_groups > 0 && (a.heads * a.vdim) % a.norm_groups == 0 && a.norm_groups <= 65535 &&
+                                       (a.norm_weight == nullptr || a.norm_weight_per_head || a.heads == 1)),
+                "linear_recurrence: a norm in %d parts of a row of %d, with a weight over the whole row", a.norm_groups, a.heads * a.vdim);
+    const int qk_rows = (a.qk_heads > 0 ? a.qk_heads : a.heads) * a.dim;
+    XRT_REQUIRE(a.q_stride >= qk_rows && a.k_stride >= qk_rows && a.v_stride >= a.heads * a.vdim &&
                 (a.gate == nullptr || a.gate_stride >= a.heads * a.vdim), "linear_recurrence: a row stride is shorter than its heads");
     XRT_REQUIRE(n_seqs >= 0 && max_count >= 0 && tokens >= 0 && tokens < (1L << 31), "linear_recurrence: bad sizes");
     if (n_seqs == 0 || tokens == 0 || max_count == 0) return 0;
@@ -519,7 +597,10 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
     if (bonus) XRT_REC_DIM(true, true); else XRT_REC_DIM(false, true);
 #undef XRT_REC_DIM
 #undef XRT_REC
-    recurrence_finish_kernel<<<dim3((unsigned)tokens, a.heads), XRT_WAVE, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
+    if (a.norm_groups > 0)
+        recurrence_finish_groups_kernel<<<dim3((unsigned)tokens, a.norm_groups), 256, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
+    else
+        recurrence_finish_kernel<<<dim3((unsigned)tokens, a.heads), XRT_WAVE, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
     XRT_LAUNCH_CHECK("linear_recurrence");
     return 0;
 }

@@ -196,6 +196,12 @@ long xrt_sample_workspace(int rows, int vocab);
 // the sequence's last taps - 1 inputs. x rows are x_stride elements apart; out is [n_out][tokens][channels] of x's type.
 // XRT_CONV_PLUS_INPUT adds x[t][c]; XRT_CONV_TOWARDS_LAST (taps 2, w [n_out][channels]) gives x + (x[t - 1] - x) * w.
 enum { XRT_CONV_PLAIN = 0, XRT_CONV_PLUS_INPUT = 1, XRT_CONV_TOWARDS_LAST = 2 };
+enum { XRT_CONV_ACT_NONE = 0, XRT_CONV_ACT_SILU = 1 };
+// The same with a bias [n_out][channels] (of the filters' type, or null) added to every sum and an activation applied to the
+// result, and with a result of a type of its own (bfloat16 of float32 inputs: the state then keeps the inputs unrounded).
+int xrt_short_conv_with(const void* x, int dtype, long tokens, long x_stride, int channels, const void* w, int w_dtype, int taps,
+                        int n_out, int mode, float* state, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
+                        void* out, int out_dtype, const void* bias, int activation, void* stream);
 int xrt_short_conv(const void* x, int dtype, long tokens, long x_stride, int channels, const void* w, int w_dtype, int taps,
                    int n_out, int mode, float* state, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
                    void* out, void* stream);
@@ -207,7 +213,13 @@ int xrt_short_conv(const void* x, int dtype, long tokens, long x_stride, int cha
 // (GIVEN), exp(-exp(z)) (EXP_NEG_EXP) or sigmoid(z)^decay_power (SIGMOID_POWER). Then, per head: o / sqrt(mean(o^2) + eps) if
 // norm, times norm_weight ([vdim] for all heads, or [heads * vdim]) if given, times gate (rows of heads x vdim of the element
 // type, through silu with XRT_GATE_SILU) if given; out rows are heads x vdim.
-enum { XRT_DECAY_PER_HEAD = 0, XRT_DECAY_GIVEN = 1, XRT_DECAY_EXP_NEG_EXP = 2, XRT_DECAY_SIGMOID_POWER = 3 };
+// XRT_DECAY_STEP: a step size per token and head, step = softplus(decay[token][head] + decay_bias[head]) with decay rows
+// decay_stride apart; all channels of the head decay by exp(-exp(decay_rate[head]) * step), and v enters the state times step.
+// qk_heads (0: as many as heads): heads of q and k; head h reads head h / (heads / qk_heads) of them. skip [heads]: o += skip * v.
+// norm_groups > 0 (with norm): the gate comes first, then the token's whole row of heads x vdim is divided by the root mean
+// square of each of its norm_groups equal parts, times norm_weight [heads * vdim]. gate_is_float32: the gate's rows are float32
+// whatever the element type.
+enum { XRT_DECAY_PER_HEAD = 0, XRT_DECAY_GIVEN = 1, XRT_DECAY_EXP_NEG_EXP = 2, XRT_DECAY_SIGMOID_POWER = 3, XRT_DECAY_STEP = 4 };
 enum { XRT_GATE_PLAIN = 0, XRT_GATE_SILU = 1 };
 typedef struct {
     const void *q, *k, *v;
@@ -230,6 +242,14 @@ typedef struct {
     long gate_stride;
     int gate_act;
     void* out;
+    long decay_stride;
+    const void* decay_rate;
+    int decay_rate_dtype;
+    int qk_heads;
+    const void* skip;
+    int skip_dtype;
+    int norm_groups;
+    int gate_is_float32;
 } xrt_recurrence;
 // token_slots [tokens]: the slot of every token's sequence. The workspace holds the raw outputs and, where a long prompt is cut
 // into segments that run side by side, the segments' states; xrt_linear_recurrence_workspace says how many floats.
@@ -258,12 +278,13 @@ int xrt_kv_store(const void* k, long k_stride, const void* v, long v_stride, int
 // q_stride: 0 (rows of qkv are q, k and v side by side), or the distance between the rows of q where they lie alone (keys and
 // values are read from the cache only). distance_bias: null, or float32 [n_heads][bias_span]: a key d tokens behind the query
 // adds distance_bias[h][min(d, bias_span - 1)] to its scaled score (any bias that is a function of head and distance and
-// stays constant from some distance on).
+// stays constant from some distance on). chunk: 0, or the size of the stretches that positions are cut into from a
+// sequence's first token on; a query then sees only the keys of its own stretch (at or before it).
 int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* positions, const int* slots, void* out, float scale, int window,
                           const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
-                          void* stream);
+                          int chunk, void* stream);
 
 // Attention without a softmax: the weight of a visible key is sigmoid(score_h + head_bias[h]), not normalised over the keys;
 // before that the heads' scaled scores of a (query, key) pair are mixed, score_h <- sum_g head_mix[h][g] score_g
@@ -310,6 +331,60 @@ int xrt_layernorm_shift(const float* x, const void* weight, const void* bias, co
 int xrt_add_layernormed(float* residual, const float* y, const void* pre_bias, const void* weight, const void* bias, int w_dtype,
                         float eps, float scale, const void* next_weight, const void* next_bias, float next_eps, void* next_out,
                         int out_dtype, long rows, int hidden, void* stream);
+
+// ---- the selective scan (csrc/selective_scan.hip) ----------------------------------------------------------------------
+// Per channel c a state [n] (float32, state [slots][channels][n]): with step = softplus(step[t][c] + step_bias[c]) of every
+// token in turn  S[c][j] <- exp(step * A[c][j]) S[c][j] + step x[t][c] b[t][j],  y = sum_j S[c][j] c[t][j] + skip[c] x[t][c],
+// A = -exp(a_log) ([channels][n]); out = y * silu(gate[t][c]) (gate may be null). x, out: element type dtype; step, b, c:
+// float32; step_bias, a_log, skip: small_dtype; gate: gate_dtype. Rows lie their strides apart; out rows are `channels` wide.
+typedef struct {
+    const void* x; long x_stride; int dtype;
+    const float* step; long step_stride;
+    const void* step_bias;
+    const float* b; long b_stride;
+    const float* c; long c_stride;
+    const void* a_log;
+    const void* skip;
+    int small_dtype;
+    const void* gate; long gate_stride; int gate_dtype;
+    float* state;
+    void* out;
+    int channels, n;
+} xrt_selective_scan_args;
+long xrt_selective_scan_workspace(int n_seqs, int max_count, long tokens, int channels, int n);
+int xrt_selective_scan(const xrt_selective_scan_args* args, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
+                       const int* token_slots, long tokens, float* workspace, long workspace_floats, void* stream);
+
+// ---- what a token brings beside its embedding row, and small operations on rows (csrc/token_inputs.hip) -----------------
+// x[t] <- x[t] * scale + table[row(t)] (x float32 [tokens][width]; table [buckets + 1][width], or null: the scale alone).
+// row(t) = (before * mul_prev + id * mul_cur) mod buckets with `before` the token before t in its sequence: the one at the
+// packed place before it if that is the same sequence's, else before[slot] (what the step before left; int32 [slots]); a
+// sequence's first token (position 0) reads row `buckets`. Afterwards before[slot] is the sequence's last token of the step.
+int xrt_bigram_add(float* x, long tokens, int width, float scale, const void* table, int table_dtype, int buckets, int mul_prev,
+                   int mul_cur, const int* ids, const int* positions, const int* slots, const int* seq_offsets,
+                   const int* seq_slots, int n_seqs, int* before, void* stream);
+// out[t][c] = gelu_tanh(s[t][c]) * table[ids[t]][offset + c] for c < width; s float32 rows s_stride apart; table [rows][table_width]
+int xrt_gated_rows(const float* s, long s_stride, const void* table, int table_dtype, long table_width, long offset, int rows,
+                   const int* ids, void* out, int out_dtype, long tokens, int width, void* stream);
+// residual += sum over n < count of scales[n] * gains[n][column] * y[n] (y float32 [rows][width]; a null gain is all ones)
+int xrt_add_weighted(float* residual, int count, const float* const* y, const void* const* gains, const float* scales, int gain_dtype,
+                     long rows, int width, void* stream);
+// out[r][c] = g * sigmoid(alpha * g) * (u + 1), g = min(sums[r][c], limit), u = clamp(sums[r][n + c], -limit, limit)
+int xrt_glu_clamped(const float* sums, void* out, int out_dtype, long rows, int n, float limit, float alpha, void* stream);
+// x <- cap * tanh(x / cap), float32 in place
+int xrt_softcap(float* x, long count, float cap, void* stream);
+int xrt_cast(const void* x, int x_dtype, void* out, int out_dtype, long count, void* stream);
+
+// ---- experts (csrc/experts.hip) --------------------------------------------------------------------------------------------
+// The choice of experts for every token from router logits [tokens][experts] (float32): scores sigmoid(z); `groups` equal
+// groups of neighbours, a group's score the sum of its group_top largest scores, experts of the `keep` best groups stay
+// open; the `top` largest open scores are chosen; weights [tokens][experts] (float32) get score / (sum of the chosen scores
+// + floor) for the chosen and 0 for the others; chosen (or null) [tokens][top] the experts in the order of their scores.
+#define XRT_MOST_EXPERTS 256
+int xrt_route_experts(const float* logits, long tokens, int experts, int top, int groups, int keep, int group_top, float floor_,
+                      float* weights, int* chosen, void* stream);
+// act[t][e * width + c] *= weights[t][e]
+int xrt_scale_blocks(void* act, int dtype, const float* weights, long tokens, int experts, int width, void* stream);
 
 #ifdef __cplusplus
 }

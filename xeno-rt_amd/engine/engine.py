@@ -73,10 +73,7 @@ class Engine:
             limit = min(limit, model_context)
         if max_slots is None:
             max_slots = max(1, min((max_tokens + BLOCK_TOKENS - 1) // BLOCK_TOKENS, MOST_SLOTS_BY_DEFAULT))
-        schedule = spec.schedule
-        reads_from = [i if call.reads_cache_of is None else call.reads_cache_of
-                      for i, call in enumerate(schedule)]
-        self.cache = SequenceCache(spec.cache_needs(), reads_from, max_tokens, max_slots, limit,
+        self.cache = SequenceCache(spec.cache_needs(), spec.cache_sources(), max_tokens, max_slots, limit,
                                    self.dtype, self.device)
         self.vocab_size = spec.head.vocab
         # decode steps are replayed as HIP graphs where the model allows it

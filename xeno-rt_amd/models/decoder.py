@@ -73,9 +73,20 @@ class ModelSpec:
         return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
 
     def cache_needs(self) -> List[Optional[CacheNeeds]]:
-        """For each schedule entry what its cache entry holds, None if it reads another's."""
-        return [None if call.reads_cache_of is not None else self.layers[call.layer].cache_needs()
-                for call in self.schedule]
+        """For each schedule entry what its cache entry holds, None if it reads another's; then, if the embedding keeps
+        something per sequence (`keeps_state`), one more entry for it."""
+        needs = [None if call.reads_cache_of is not None else self.layers[call.layer].cache_needs()
+                 for call in self.schedule]
+        if getattr(self.embedding, "keeps_state", False):
+            needs.append(self.embedding.cache_needs())
+        return needs
+
+    def cache_sources(self) -> List[int]:
+        """For each entry of `cache_needs` the entry whose storage it reads: itself, unless the schedule says otherwise."""
+        sources = [index if call.reads_cache_of is None else call.reads_cache_of for index, call in enumerate(self.schedule)]
+        if getattr(self.embedding, "keeps_state", False):
+            sources.append(len(sources))
+        return sources
 
 
 class DecoderModel:
@@ -91,7 +102,10 @@ class DecoderModel:
     def forward(self, batch, cache) -> torch.Tensor:
         """Logits [len(batch.logit_rows), vocab] in float32 for the tokens of `batch`."""
         spec = self.spec
-        x = spec.embedding.forward(batch.token_ids, batch.positions)
+        if getattr(spec.embedding, "keeps_state", False):       # its cache entry follows the schedule's
+            x = spec.embedding.forward_step(batch, cache.layer_cache(len(spec.schedule)))
+        else:
+            x = spec.embedding.forward(batch.token_ids, batch.positions)
         h = None            # the next block's first norm of x, where the block before it has made it already
         for index, call in enumerate(spec.schedule):
             block = spec.layers[call.layer]

@@ -133,11 +133,25 @@ class _Recurrence(ctypes.Structure):
                 ("decay_power", ctypes.c_float), ("bonus", ctypes.c_void_p), ("bonus_dtype", ctypes.c_int),
                 ("state", ctypes.c_void_p), ("norm", ctypes.c_int), ("eps", ctypes.c_float),
                 ("norm_weight", ctypes.c_void_p), ("norm_weight_dtype", ctypes.c_int), ("norm_weight_per_head", ctypes.c_int),
-                ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_long), ("gate_act", ctypes.c_int), ("out", ctypes.c_void_p)]
+                ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_long), ("gate_act", ctypes.c_int), ("out", ctypes.c_void_p),
+                ("decay_stride", ctypes.c_long), ("decay_rate", ctypes.c_void_p), ("decay_rate_dtype", ctypes.c_int),
+                ("qk_heads", ctypes.c_int), ("skip", ctypes.c_void_p), ("skip_dtype", ctypes.c_int),
+                ("norm_groups", ctypes.c_int), ("gate_is_float32", ctypes.c_int)]
+
+
+class _SelectiveScan(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("x_stride", ctypes.c_long), ("dtype", ctypes.c_int),
+                ("step", ctypes.c_void_p), ("step_stride", ctypes.c_long), ("step_bias", ctypes.c_void_p),
+                ("b", ctypes.c_void_p), ("b_stride", ctypes.c_long), ("c", ctypes.c_void_p), ("c_stride", ctypes.c_long),
+                ("a_log", ctypes.c_void_p), ("skip", ctypes.c_void_p), ("small_dtype", ctypes.c_int),
+                ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_long), ("gate_dtype", ctypes.c_int),
+                ("state", ctypes.c_void_p), ("out", ctypes.c_void_p), ("channels", ctypes.c_int), ("n", ctypes.c_int)]
 
 
 CONV_MODES = {"plain": 0, "plus_input": 1, "towards_last": 2}          # XRT_CONV_* of the library
-DECAY_MODES = {"per_head": 0, "given": 1, "exp_neg_exp": 2, "sigmoid_power": 3}      # XRT_DECAY_*
+DECAY_MODES = {"per_head": 0, "given": 1, "exp_neg_exp": 2, "sigmoid_power": 3, "step": 4}      # XRT_DECAY_*
+CONV_ACTIVATIONS = {None: 0, "silu": 1}                                # XRT_CONV_ACT_*
+MOST_EXPERTS = 256                                                     # XRT_MOST_EXPERTS
 UNARY = {"tanh": 0, "silu": 1, "xielu": 2}                             # XRT_UNARY_*
 
 
@@ -182,7 +196,9 @@ class HipOps:
                      "xrt_attention_finishes_qkv", "xrt_attention_finishing", "xrt_rope_table", "xrt_short_conv",
                      "xrt_linear_recurrence", "xrt_add_normed", "xrt_activation", "xrt_rows_add", "xrt_kv_store",
                      "xrt_attention_general", "xrt_rmsnorm_conv_step", "xrt_attention_sigmoid", "xrt_qkv_complete",
-                     "xrt_layernorm", "xrt_layernorm_shift", "xrt_add_layernormed"):
+                     "xrt_layernorm", "xrt_layernorm_shift", "xrt_add_layernormed", "xrt_short_conv_with", "xrt_selective_scan",
+                     "xrt_bigram_add", "xrt_gated_rows", "xrt_add_weighted", "xrt_glu_clamped", "xrt_softcap", "xrt_cast",
+                     "xrt_route_experts", "xrt_scale_blocks"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -195,6 +211,7 @@ class HipOps:
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
         self.lib.xrt_linear_recurrence_workspace.restype = ctypes.c_long
         self.lib.xrt_attention_sigmoid_workspace.restype = ctypes.c_long
+        self.lib.xrt_selective_scan_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -467,8 +484,9 @@ class HipOps:
 
     def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None,
                   finish: Optional[QkvFinish] = None, value_dim: Optional[int] = None, sink: bool = False,
-                  distance_bias: Optional[torch.Tensor] = None, queries_alone: bool = False):
-        """Causal attention of the step's tokens over the cache. distance_slopes: float32 [n_heads], or None; a key at
+                  distance_bias: Optional[torch.Tensor] = None, queries_alone: bool = False, chunk: Optional[int] = None):
+        """Causal attention of the step's tokens over the cache. chunk: positions are cut into stretches of this many from a
+        sequence's first token on, and a query sees the keys of its own stretch only. distance_slopes: float32 [n_heads], or None; a key at
         position j adds slope * (j - P) to the scaled score of the query at position P. distance_bias: float32
         [n_heads, span], or None; a key d tokens behind the query adds distance_bias[h, min(d, span - 1)]. queries_alone: the
         rows of `qkv` hold the queries only (keys and values are in the cache already). finish: what is still to do to
@@ -476,9 +494,9 @@ class HipOps:
         from ..cache import BLOCK_TOKENS
         if finish is not None:
             return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
-        if sink or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone:
+        if sink or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone or chunk:
             return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
-                                           distance_slopes, sink, distance_bias, queries_alone)
+                                           distance_slopes, sink, distance_bias, queries_alone, chunk)
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -513,7 +531,7 @@ class HipOps:
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
     def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink,
-                           distance_bias=None, queries_alone=False):
+                           distance_bias=None, queries_alone=False, chunk=None):
         """Rows of qkv are [n_heads x head_dim | n_kv_heads x head_dim | n_kv_heads x value_dim] (or the queries alone), rows of
         out n_heads x value_dim. sink: the softmax's denominator has one more (a key of score 0 without a value)."""
         tokens = qkv.shape[0]
@@ -535,7 +553,8 @@ class HipOps:
         self._check(self.lib.xrt_attention_general(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, value_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table), stride,
             n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale), int(window or 0),
-            _ptr(distance_slopes), int(bool(sink)), ctypes.c_long(q_stride), _ptr(distance_bias), int(span), self._stream(qkv)))
+            _ptr(distance_slopes), int(bool(sink)), ctypes.c_long(q_stride), _ptr(distance_bias), int(span), int(chunk or 0),
+            self._stream(qkv)))
 
     def attention_sigmoid(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window=None, head_mix=None,
                           head_bias=None, gate=None):
@@ -695,7 +714,7 @@ class HipOps:
             raise KernelError(f"the step has {batch.n_tokens} tokens, the operand {tokens} rows")
         return _ptr(batch.sequence_offsets), _ptr(batch.sequence_slots), n
 
-    def short_conv(self, x, w, state, batch, out, mode="plain"):
+    def short_conv(self, x, w, state, batch, out, mode="plain", bias=None, activation=None):
         """out[o, t, c] = sum_j w[o, c, j] x[t - taps + 1 + j, c] along each sequence; state [slots, taps - 1, channels] (float32)
         holds what came before the step and is brought up to date. w is [channels, taps] or [n_out, channels, taps]; mode
         "plus_input" adds x, "towards_last" (w [n_out, channels], two taps) gives x + (x[t - 1] - x) * w."""
@@ -710,11 +729,13 @@ class HipOps:
             taps, n_out = w.shape[-1], (1 if w.dim() == 2 else w.shape[0])
             self._require(w, "short_conv w", None, (channels, taps) if w.dim() == 2 else (n_out, channels, taps), x)
         self._require(state, "short_conv state", torch.float32, (state.shape[0], taps - 1, channels), x)
-        self._require(out, "short_conv out", x.dtype, (tokens, channels) if out.dim() == 2 and n_out == 1 else (n_out, tokens, channels), x)
+        self._require(out, "short_conv out", None, (tokens, channels) if out.dim() == 2 and n_out == 1 else (n_out, tokens, channels), x)
+        if bias is not None:
+            self._require(bias, "short_conv bias", w.dtype, (channels,) if n_out == 1 and bias.dim() == 1 else (n_out, channels), x)
         offsets, slots, n = self._sequences(batch, tokens, x)
-        self._check(self.lib.xrt_short_conv(_ptr(x), _code(x), ctypes.c_long(tokens), ctypes.c_long(stride), channels, _ptr(w), _code(w), taps,
-                                            n_out, CONV_MODES[mode], _ptr(state), offsets, slots, n, int(batch.max_count), _ptr(out),
-                                            self._stream(x)))
+        self._check(self.lib.xrt_short_conv_with(_ptr(x), _code(x), ctypes.c_long(tokens), ctypes.c_long(stride), channels, _ptr(w), _code(w),
+                                                 taps, n_out, CONV_MODES[mode], _ptr(state), offsets, slots, n, int(batch.max_count),
+                                                 _ptr(out), _code(out), _ptr(bias), CONV_ACTIVATIONS[activation], self._stream(x)))
 
     def rmsnorm_conv_step(self, x, weight, eps, conv_w, state, batch, out, plus_input=False):
         """`rmsnorm` of the rows of x, then `short_conv` of the normed rows (plain or plus the input), in one kernel and to the
@@ -735,16 +756,23 @@ class HipOps:
 
     def linear_recurrence(self, q, k, v, state, batch, out, heads, dim, vdim, decay, decay_mode="per_head", decay_bias=None,
                           decay_power=1.0, q_scale=1.0, k_scale=1.0, bonus=None, norm_eps=None, norm_weight=None, gate=None,
-                          gate_activation="silu"):
+                          gate_activation="silu", decay_rate=None, qk_heads=None, skip=None, norm_groups=None):
         """Per sequence and head S <- diag(decay) S + k v^T, o = S^T q (with `bonus` [heads, dim]: o = (S + diag(bonus) k v^T)^T q
         before the update); state [slots, heads, dim, vdim] float32. decay: float32 [heads] ("per_head") or [tokens, heads * dim]
         ("given": the decay itself; "exp_neg_exp": exp(-exp(z + bias)); "sigmoid_power": sigmoid(z + bias)^decay_power). Then per head
         o / sqrt(mean(o^2) + norm_eps) (if norm_eps is given), times norm_weight ([vdim] or [heads * vdim]), times gate
-        (through silu, or "plain")."""
+        (through silu, or "plain"; the gate's rows may be float32 beside bfloat16 operands).
+        decay_mode "step": decay is float32 [tokens, heads] (columns of a wider matrix will do), a step size softplus(z + bias)
+        per token and head with decay_bias [heads]; the head's channels all decay by exp(-exp(decay_rate[head]) * step) and v
+        enters the state times the step. qk_heads: q and k have this many heads, shared by neighbouring heads in equal groups.
+        skip [heads]: o += skip * v. norm_groups: the gate comes before the norm, which then spans each of that many equal
+        parts of the token's whole row, with norm_weight [heads * vdim]."""
         tokens = q.shape[0]
         record = _Recurrence()
-        record.q_stride = self._rows(q, "recurrence q", heads * dim)
-        record.k_stride = self._rows(k, "recurrence k", heads * dim, q.dtype, q)
+        qk = heads if qk_heads is None else int(qk_heads)
+        record.qk_heads = qk
+        record.q_stride = self._rows(q, "recurrence q", qk * dim)
+        record.k_stride = self._rows(k, "recurrence k", qk * dim, q.dtype, q)
         record.v_stride = self._rows(v, "recurrence v", heads * vdim, q.dtype, q)
         record.q, record.k, record.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
         record.heads, record.dim, record.vdim = heads, dim, vdim
@@ -752,10 +780,22 @@ class HipOps:
         if decay_mode not in DECAY_MODES:
             raise KernelError(f"linear_recurrence: decay_mode must be one of {sorted(DECAY_MODES)}")
         record.decay_mode = DECAY_MODES[decay_mode]
-        self._require(decay, "recurrence decay", torch.float32, (heads,) if decay_mode == "per_head" else (tokens, heads * dim), q)
+        if decay_mode == "step":
+            record.decay_stride = self._rows(decay, "recurrence steps", heads, torch.float32, q)
+            if decay_rate is None:
+                raise KernelError("linear_recurrence: decays from step sizes need a rate per head")
+            self._require(decay_rate, "recurrence decay_rate", None, (heads,), q)
+            record.decay_rate, record.decay_rate_dtype = decay_rate.data_ptr(), _code(decay_rate)
+        else:
+            self._require(decay, "recurrence decay", torch.float32, (heads,) if decay_mode == "per_head" else (tokens, heads * dim), q)
         record.decay = decay.data_ptr()
+        if skip is not None:
+            self._require(skip, "recurrence skip", None, (heads,), q)
+            record.skip, record.skip_dtype = skip.data_ptr(), _code(skip)
+        if norm_groups is not None:
+            record.norm_groups = int(norm_groups)
         if decay_bias is not None:
-            self._require(decay_bias, "recurrence decay_bias", None, (heads * dim,), q)
+            self._require(decay_bias, "recurrence decay_bias", None, (heads,) if decay_mode == "step" else (heads * dim,), q)
             record.decay_bias, record.decay_bias_dtype = decay_bias.data_ptr(), _code(decay_bias)
         record.decay_power = float(decay_power)
         if bonus is not None:
@@ -771,7 +811,10 @@ class HipOps:
             record.norm_weight, record.norm_weight_dtype = norm_weight.data_ptr(), _code(norm_weight)
             record.norm_weight_per_head = int(tuple(norm_weight.shape) == (heads * vdim,) and heads > 1)
         if gate is not None:
-            record.gate_stride = self._rows(gate, "recurrence gate", heads * vdim, q.dtype, q)
+            record.gate_stride = self._rows(gate, "recurrence gate", heads * vdim, None, q)
+            if gate.dtype not in (q.dtype, torch.float32):
+                raise KernelError(f"recurrence gate: dtype {gate.dtype}, expected {q.dtype} or float32")
+            record.gate_is_float32 = int(gate.dtype == torch.float32)
             record.gate, record.gate_act = gate.data_ptr(), {"plain": 0, "silu": 1}[gate_activation]
         self._require(out, "recurrence out", q.dtype, (tokens, heads * vdim), q)
         record.out = out.data_ptr()
@@ -782,6 +825,127 @@ class HipOps:
         self._check(self.lib.xrt_linear_recurrence(ctypes.byref(record), _code(q), offsets, slots, n, int(batch.max_count),
                                                    _ptr(batch.slots), ctypes.c_long(tokens), _ptr(workspace), ctypes.c_long(need),
                                                    self._stream(q)))
+
+    def selective_scan(self, x, step, b, c, state, batch, out, a_log, step_bias=None, skip=None, gate=None):
+        """Per sequence and channel S[c, :] <- exp(dt A[c, :]) S[c, :] + dt x[t, c] b[t, :], y = S[c, :] . c[t, :] + skip[c] x[t, c],
+        with dt = softplus(step[t, c] + step_bias[c]) and A = -exp(a_log) [channels, n]; out = y * silu(gate). x and out have
+        the compute dtype; step [tokens, channels], b and c [tokens, n] are float32 (columns of wider matrices will do); state
+        [slots, channels, n] float32; gate compute dtype or float32."""
+        tokens, channels = x.shape
+        n = a_log.shape[1]
+        record = _SelectiveScan()
+        record.x_stride, record.dtype, record.x = self._rows(x, "selective_scan x"), _code(x), x.data_ptr()
+        record.step_stride, record.step = self._rows(step, "selective_scan step", channels, torch.float32, x), step.data_ptr()
+        record.b_stride, record.b = self._rows(b, "selective_scan b", n, torch.float32, x), b.data_ptr()
+        record.c_stride, record.c = self._rows(c, "selective_scan c", n, torch.float32, x), c.data_ptr()
+        self._require(a_log, "selective_scan a_log", None, (channels, n), x)
+        record.a_log, record.small_dtype = a_log.data_ptr(), _code(a_log)
+        for what, tensor in (("step_bias", step_bias), ("skip", skip)):
+            if tensor is not None:
+                self._require(tensor, f"selective_scan {what}", a_log.dtype, (channels,), x)
+                setattr(record, what, tensor.data_ptr())
+        if gate is not None:
+            record.gate_stride, record.gate_dtype, record.gate = self._rows(gate, "selective_scan gate", channels, None, x), _code(gate), gate.data_ptr()
+        self._require(state, "selective_scan state", torch.float32, (state.shape[0], channels, n), x)
+        self._require(out, "selective_scan out", x.dtype, (tokens, channels), x)
+        record.state, record.out, record.channels, record.n = state.data_ptr(), out.data_ptr(), channels, n
+        offsets, slots, n_seqs = self._sequences(batch, tokens, x)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), x)
+        need = int(self.lib.xrt_selective_scan_workspace(n_seqs, int(batch.max_count), ctypes.c_long(tokens), channels, n))
+        workspace = self._empty(need, torch.float32, x.device) if need > 0 else None
+        self._check(self.lib.xrt_selective_scan(ctypes.byref(record), offsets, slots, n_seqs, int(batch.max_count), _ptr(batch.slots),
+                                                ctypes.c_long(tokens), _ptr(workspace), ctypes.c_long(need), self._stream(x)))
+
+    def bigram_add(self, x, scale, batch, table=None, before=None, buckets=0, mul_prev=0, mul_cur=0):
+        """x <- x * scale + table[row]: row (token before * mul_prev + token * mul_cur) mod buckets, row `buckets` for a sequence's
+        first token; before [slots] (int32) holds every sequence's last token of the step before and is brought up to date."""
+        tokens, width = x.shape
+        self._require(x, "bigram_add x", torch.float32)
+        n_seqs = 0
+        offsets = seq_slots = None
+        if table is not None:
+            self._require(table, "bigram_add table", None, (buckets + 1, width), x)
+            self._require(before, "bigram_add before", torch.int32, None, x)
+            self._require(batch.token_ids, "token ids", torch.int32, (tokens,), x)
+            self._require(batch.positions, "positions", torch.int32, (tokens,), x)
+            self._require(batch.slots, "slots", torch.int32, (tokens,), x)
+            offsets, seq_slots, n_seqs = self._sequences(batch, tokens, x)
+        self._check(self.lib.xrt_bigram_add(_ptr(x), ctypes.c_long(tokens), width, ctypes.c_float(scale), _ptr(table),
+                                            0 if table is None else _code(table), int(buckets), int(mul_prev), int(mul_cur),
+                                            _ptr(batch.token_ids), _ptr(batch.positions), _ptr(batch.slots), offsets, seq_slots, n_seqs,
+                                            _ptr(before), self._stream(x)))
+
+    def gated_rows(self, s, table, ids, offset, out):
+        """out[t, c] = gelu_tanh(s[t, c]) * table[ids[t], offset + c]; s float32 [tokens, width]."""
+        tokens, width = s.shape
+        stride = self._rows(s, "gated_rows s", None, torch.float32)
+        self._require(table, "gated_rows table", None, None, s)
+        self._require(ids, "gated_rows ids", torch.int32, (tokens,), s)
+        self._require(out, "gated_rows out", None, (tokens, width), s)
+        if table.dim() != 2 or offset < 0 or offset + width > table.shape[1]:
+            raise KernelError(f"gated_rows: columns {offset} to {offset + width} of a table {tuple(table.shape)}")
+        self._check(self.lib.xrt_gated_rows(_ptr(s), ctypes.c_long(stride), _ptr(table), _code(table), ctypes.c_long(table.shape[1]),
+                                            ctypes.c_long(offset), table.shape[0], _ptr(ids), _ptr(out), _code(out), ctypes.c_long(tokens),
+                                            width, self._stream(s)))
+
+    def add_weighted(self, residual, terms):
+        """residual += sum over (y, gain, scale) in terms of scale * gain * y; y float32 like residual, gain [width] or None; one to
+        four terms."""
+        self._require(residual, "add_weighted residual", torch.float32)
+        if residual.dim() != 2 or not 1 <= len(terms) <= 4:
+            raise KernelError("add_weighted: a residual [rows, width] and one to four terms")
+        rows, width = residual.shape
+        gains = [gain for _, gain, _ in terms if gain is not None]
+        for y, gain, _ in terms:
+            self._require(y, "add_weighted y", torch.float32, (rows, width), residual)
+            if gain is not None:
+                self._require(gain, "add_weighted gain", gains[0].dtype, (width,), residual)
+        count = len(terms)
+        ys = (ctypes.c_void_p * count)(*[y.data_ptr() for y, _, _ in terms])
+        gs = (ctypes.c_void_p * count)(*[0 if gain is None else gain.data_ptr() for _, gain, _ in terms])
+        scales = (ctypes.c_float * count)(*[float(scale) for _, _, scale in terms])
+        self._check(self.lib.xrt_add_weighted(_ptr(residual), count, ys, gs, scales, _code(gains[0]) if gains else 0, ctypes.c_long(rows),
+                                              width, self._stream(residual)))
+
+    def glu_clamped(self, sums, out, limit, alpha):
+        """out = g * sigmoid(alpha g) * (u + 1) with g = min(sums[:, :n], limit), u = clamp(sums[:, n:], -limit, limit)."""
+        rows, n = out.shape
+        self._require(sums, "glu_clamped sums", torch.float32, (rows, 2 * n))
+        self._require(out, "glu_clamped out", None, (rows, n), sums)
+        self._check(self.lib.xrt_glu_clamped(_ptr(sums), _ptr(out), _code(out), ctypes.c_long(rows), n, ctypes.c_float(limit),
+                                             ctypes.c_float(alpha), self._stream(sums)))
+
+    def softcap(self, x, cap):
+        """x <- cap * tanh(x / cap), in place; x float32."""
+        self._require(x, "softcap x", torch.float32)
+        self._check(self.lib.xrt_softcap(_ptr(x), ctypes.c_long(x.numel()), ctypes.c_float(cap), self._stream(x)))
+
+    def cast(self, x, out):
+        """out = x in out's element type."""
+        self._require(x, "cast x")
+        self._require(out, "cast out", None, x.shape, x)
+        self._check(self.lib.xrt_cast(_ptr(x), _code(x), _ptr(out), _code(out), ctypes.c_long(x.numel()), self._stream(x)))
+
+    def route_experts(self, logits, weights, top, groups=1, keep=1, group_top=2, floor=1e-20, chosen=None):
+        """From router logits [tokens, experts] (float32) the weights [tokens, experts] (float32; zero for experts not chosen):
+        scores sigmoid(z); experts in `groups` equal groups of neighbours, a group's score the sum of its group_top largest,
+        experts of the `keep` best groups stay open; the `top` largest open scores are chosen and divided by their sum + floor.
+        chosen (int32 [tokens, top], or None) takes the chosen experts in the order of their scores."""
+        tokens, experts = logits.shape
+        self._require(logits, "route_experts logits", torch.float32)
+        self._require(weights, "route_experts weights", torch.float32, (tokens, experts), logits)
+        if chosen is not None:
+            self._require(chosen, "route_experts chosen", torch.int32, (tokens, top), logits)
+        self._check(self.lib.xrt_route_experts(_ptr(logits), ctypes.c_long(tokens), experts, int(top), int(groups), int(keep), int(group_top),
+                                               ctypes.c_float(floor), _ptr(weights), _ptr(chosen), self._stream(logits)))
+
+    def scale_blocks(self, act, weights, width):
+        """act[t, e * width + c] *= weights[t, e], in place."""
+        tokens, experts = weights.shape
+        self._require(weights, "scale_blocks weights", torch.float32)
+        self._require(act, "scale_blocks act", None, (tokens, experts * width), weights)
+        self._check(self.lib.xrt_scale_blocks(_ptr(act), _code(act), _ptr(weights), ctypes.c_long(tokens), experts, int(width),
+                                              self._stream(act)))
 
     def add_normed(self, residual, parts, eps, scale=1.0):
         """residual += scale * sum over (x, gain) in parts of x / sqrt(mean(x^2) + eps) * gain; x float32 like residual; one or two parts."""

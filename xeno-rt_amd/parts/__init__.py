@@ -1,15 +1,15 @@
 """Parts that models are built from."""
 from .base import (Block, CacheNeeds, FeedForward, HalfSplitRotation, KVSpec, Mixer, Norm, Part, PositionEncoding,
                    Runtime, StateSpec, WeightSpec, create_part, register_part, registered_parts)
-from .norm import LayerNorm, RMSNorm, ScalarRMSNorm
+from .norm import LayerNorm, OffsetRMSNorm, RMSNorm, ScalarRMSNorm
 from .position import DistanceBuckets, DistanceSlopes, NoPosition, PairRotation, Rotary
 from .convolution import ShortConvolution, TokenShift
 from .attention import Attention, SharedValues
-from .recurrent import GatedLinearAttention, Retention, TimeMixWKV
-from .parallel import ParallelMixer
-from .feedforward import DenseMLP, GatedMLP
-from .block import PreNormBlock, SandwichBlock
-from .embedding import Embedding, OutputHead, PositionedEmbedding
+from .recurrent import GatedLinearAttention, Retention, SelectiveStateSpace, StateSpaceDuality, TimeMixWKV
+from .parallel import ParallelMixer, WeightedPair
+from .feedforward import ClampedGLU, DenseMLP, ExpertsMLP, GatedMLP
+from .block import ParallelBlock, PreNormBlock, SandwichBlock
+from .embedding import Embedding, HashedPairEmbedding, OutputHead, PositionedEmbedding, TokenSideInput, TokenSideTable
 
 __all__ = [
     "Block", "CacheNeeds", "FeedForward", "HalfSplitRotation", "KVSpec", "Mixer", "Norm", "Part", "PositionEncoding",
@@ -17,5 +17,6 @@ __all__ = [
     "RMSNorm", "NoPosition", "Rotary", "Attention", "GatedMLP", "PreNormBlock", "Embedding", "OutputHead",
     "ScalarRMSNorm", "DistanceSlopes", "ShortConvolution", "TokenShift", "GatedLinearAttention", "Retention", "TimeMixWKV",
     "ParallelMixer", "DenseMLP", "PositionedEmbedding", "LayerNorm", "DistanceBuckets", "PairRotation", "SharedValues",
-    "SandwichBlock",
+    "SandwichBlock", "OffsetRMSNorm", "SelectiveStateSpace", "StateSpaceDuality", "WeightedPair", "ClampedGLU", "ExpertsMLP",
+    "ParallelBlock", "HashedPairEmbedding", "TokenSideInput", "TokenSideTable",
 ]

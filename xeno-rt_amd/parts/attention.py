@@ -28,7 +28,9 @@ matrix (`head_mix`) and a number per head added (`score_bias`) before the sigmoi
 heads' outputs, sigmoid of a projection of the mixer's input (`output_gate`); values blended with those that another
 attention layer made of the same token, v <- (1 - lambda) v + lambda v_other (`values=SharedValues.source()` in the
 layer whose values are kept for the step, `.reader(name)` in those that blend them in, lambda the tensor `name`); a
-position encoding that says `pair_rotation()`, or one that says `score_bias_table()`.
+position encoding that says `pair_rotation()`, or one that says `score_bias_table()`; positions cut into stretches of
+`chunk` from a sequence's first token on, a query seeing the keys of its own stretch only; or `completed=True`, which
+asks for this path outright (float32 sums of the projection, whatever else the layer has).
 """
 from __future__ import annotations
 
@@ -69,7 +71,7 @@ class Attention(Mixer):
                  window: Optional[int] = None, value_dim: Optional[int] = None, sink: bool = False,
                  convolution=None, names: Optional[Dict[str, str]] = None, biases: bool = False, weights: str = "softmax",
                  head_mix: Optional[str] = None, score_bias: Optional[str] = None, output_gate: Optional[str] = None,
-                 values=None, unread=()):
+                 values=None, unread=(), chunk: Optional[int] = None, completed: bool = False):
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
             raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
         if weights not in ("softmax", "sigmoid"):
@@ -83,7 +85,10 @@ class Attention(Mixer):
         self.head_mix_name, self.score_bias_name, self.gate_name = head_mix, score_bias, output_gate
         self.values = values
         self.unread = tuple(unread)         # tensors under the prefix that a checkpoint may carry and this layer does not read
-        self.completed = (self.biases or weights == "sigmoid" or output_gate is not None or values is not None
+        self.chunk = None if chunk is None else int(chunk)      # positions in stretches of this many; a query sees its own stretch only
+        if self.chunk is not None and (self.chunk <= 0 or weights != "softmax"):
+            raise ValueError("stretches of positions have a positive size and are served for softmax weights")
+        self.completed = (bool(completed) or self.biases or weights == "sigmoid" or output_gate is not None or values is not None or self.chunk is not None
                           or hasattr(position, "pair_rotation") or hasattr(position, "score_bias_table"))
         if self.completed and (self.sink or convolution is not None):
             raise ValueError("the completed path of attention has neither sink nor convolution")
@@ -252,7 +257,7 @@ class Attention(Mixer):
         table = self.position.score_bias_table() if hasattr(self.position, "score_bias_table") else None
         slopes = None if self.position is None else self.position.score_slopes()
         ops.attention(q, self.n_heads, self.n_kv_heads, self.head_dim, cache.kv, batch, out, scale=self.scale, window=self.window,
-                      distance_slopes=slopes, value_dim=self.value_dim, distance_bias=table, queries_alone=True)
+                      distance_slopes=slopes, value_dim=self.value_dim, distance_bias=table, queries_alone=True, chunk=self.chunk)
         return out
 
     def forward_into(self, h, batch, cache, out: torch.Tensor, bias_later: bool = False):

@@ -122,7 +122,7 @@ class SandwichBlock(Block):
         return specs
 
     def ignored_names(self):
-        return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
+        return self.unread + [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
 
     def cache_needs(self) -> CacheNeeds:
         return self.mixer.cache_needs().merged(*([self.mixer_input.cache_needs()] if self.mixer_input is not None else []))
@@ -155,5 +155,68 @@ class SandwichBlock(Block):
         self.feed_forward_post_norm.add_to(x, y, self.residual_scale)
 
 
+class ParallelBlock(Block):
+    """One norm, and both sublayers read its output: with h = norm(x), x += a * mixer(h) + b * feed_forward(h), where a and b
+    are vectors over the model width (`mixer_scale`, `feed_forward_scale`: tensor names, or None for ones). The sublayers
+    write their float32 outputs aside and one pass adds them to the stream; a mixer that is itself a weighted sum of
+    mixers (`forward_terms`) has its terms added in that same pass. `after`, if given, is a part that then adds what the
+    step's tokens bring to the stream of their own (`forward(x, batch)`)."""
+
+    def __init__(self, norm, mixer, feed_forward=None, hidden=None, mixer_scale=None, feed_forward_scale=None, after=None):
+        self.norm, self.mixer, self.feed_forward, self.after = norm, mixer, feed_forward, after
+        self.hidden = int(hidden if hidden is not None else norm.dim)
+        self.scale_names = (mixer_scale, feed_forward_scale if feed_forward is not None else None)
+        self.unread = [feed_forward_scale] if feed_forward is None and feed_forward_scale is not None else []
+        self.scales = [None, None]
+
+    def parts(self):
+        return tuple(part for part in (self.norm, self.mixer, self.feed_forward, self.after) if part is not None)
+
+    @property
+    def capturable(self) -> bool:
+        return all(part.capturable for part in self.parts())
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        specs: Dict[str, WeightSpec] = {name: WeightSpec((self.hidden,), init="ones", kind="vector")
+                                        for name in self.scale_names if name is not None}
+        for part in self.parts():
+            specs.update(part.weight_specs())
+        return specs
+
+    def ignored_names(self):
+        return self.unread + [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
+
+    def cache_needs(self) -> CacheNeeds:
+        return self.mixer.cache_needs()
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        for part in self.parts():
+            part.bind(tensors, runtime)
+        # (float32 whatever the file stores: the sum onto the stream is float32, and the gains of one pass share a type)
+        self.scales = [None if name is None else runtime.vector(tensors[name]).to(torch.float32) for name in self.scale_names]
+
+    def first_norm(self):
+        return self.norm
+
+    def forward(self, x, batch, cache) -> None:
+        rt = self.runtime
+        h = self.norm.forward(x)
+        if hasattr(self.mixer, "forward_terms"):
+            terms = [(y, self.scales[0], scale) for y, scale in self.mixer.forward_terms(h, batch, cache, x)]
+        else:
+            y = rt.empty(x.shape, torch.float32)
+            self.mixer.forward_into(h, batch, cache, y)
+            terms = [(y, self.scales[0], 1.0)]
+        if self.feed_forward is not None:
+            y = rt.empty(x.shape, torch.float32)
+            self.feed_forward.forward_into(h, batch, y)
+            terms.append((y, self.scales[1], 1.0))
+        rt.ops.add_weighted(x, terms)
+        if self.after is not None:
+            self.after.forward(x, batch)
+
+
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "sandwich", SandwichBlock)

@@ -15,10 +15,13 @@ from .base import CacheNeeds, Part, Runtime, StateSpec, WeightSpec
 class ShortConvolution(Part):
     """y[t] = sum_j w[:, j] * u[t - taps + 1 + j] on every channel, zeros before the sequence's start; with
     plus_input the result is u + y. `names` are the filters' tensors ([channels_i, taps] each), side by side along
-    the channels in the order given (so one pass serves the q, k and v of an attention)."""
+    the channels in the order given (so one pass serves the q, k and v of an attention). `bias_names`: a tensor [channels_i]
+    beside every filter, added to the sum; `activation` ("silu") is applied last. The inputs may be float32 beside a
+    compute dtype of bfloat16 (a product's sums): the state then keeps them unrounded, and the result is rounded once."""
     capturable = True
 
-    def __init__(self, names: Sequence[str], channels: Sequence[int], taps: int, state_name: str, plus_input: bool = False):
+    def __init__(self, names: Sequence[str], channels: Sequence[int], taps: int, state_name: str, plus_input: bool = False,
+                 bias_names: Sequence[str] = (), activation=None):
         if taps < 1:
             raise ValueError(f"a convolution over time needs at least one tap, found {taps}")
         self.names, self.channel_counts = list(names), [int(c) for c in channels]
@@ -26,10 +29,15 @@ class ShortConvolution(Part):
         self.taps = int(taps)
         self.state_name = state_name
         self.plus_input = plus_input
-        self.weight = None
+        self.bias_names, self.activation = list(bias_names), activation
+        if self.bias_names and len(self.bias_names) != len(self.names):
+            raise ValueError("a convolution's biases come one for every filter")
+        self.weight = self.bias = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {name: WeightSpec((count, self.taps), kind="vector") for name, count in zip(self.names, self.channel_counts)}
+        specs = {name: WeightSpec((count, self.taps), kind="vector") for name, count in zip(self.names, self.channel_counts)}
+        specs.update({name: WeightSpec((count,), init="zeros", kind="vector") for name, count in zip(self.bias_names, self.channel_counts)})
+        return specs
 
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds(states=((self.state_name, StateSpec((self.taps - 1, self.channels))),))
@@ -37,11 +45,14 @@ class ShortConvolution(Part):
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         self.weight = torch.cat([runtime.vector(tensors[name]) for name in self.names]).contiguous()
+        if self.bias_names:
+            self.bias = torch.cat([runtime.vector(tensors[name]) for name in self.bias_names]).to(self.weight.dtype).contiguous()
 
     def forward(self, u: torch.Tensor, batch, cache) -> torch.Tensor:
-        out = self.runtime.empty((u.shape[0], self.channels), u.dtype)
+        out = self.runtime.empty((u.shape[0], self.channels))
+        extra = {} if self.bias is None and self.activation is None else {"bias": self.bias, "activation": self.activation}
         self.runtime.ops.short_conv(u, self.weight, cache.states[self.state_name], batch, out,
-                                    mode="plus_input" if self.plus_input else "plain")
+                                    mode="plus_input" if self.plus_input else "plain", **extra)
         return out
 
 
@@ -51,7 +62,7 @@ class ShortConvolution(Part):
         rt = self.runtime
         scale = norm.row_scale()
         fused = getattr(rt.ops, "rmsnorm_conv_step", None)
-        if (fused is None or scale is None or len(self.names) != 1 or int(batch.max_count) != 1
+        if (fused is None or scale is None or len(self.names) != 1 or self.bias is not None or self.activation is not None or int(batch.max_count) != 1
                 or int(batch.n_tokens) != int(batch.n_sequences) or x.shape[1] != self.channels or self.taps > 8):
             return self.forward(norm.forward(x), batch, cache)
         out = rt.empty((x.shape[0], self.channels))

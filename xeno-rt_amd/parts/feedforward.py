@@ -103,5 +103,112 @@ class DenseMLP(FeedForward):
         rt.ops.linear(act, self.w_down, residual, accumulate=True)
 
 
+class ClampedGLU(FeedForward):
+    """W_down (g sigmoid(alpha g) (u + 1)) with g = min(W_gate y, limit) and u = clamp(W_up y, -limit, limit); no biases.
+    Gate and up are one product with float32 sums; the clamps and the activation read those and round once."""
+    capturable = True
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, limit: float, alpha: float = 1.702,
+                 gate: str = "gate", up: str = "up", down: str = "down"):
+        if limit <= 0:
+            raise ValueError(f"the clamp's limit must be positive, found {limit}")
+        self.hidden, self.intermediate, self.limit, self.alpha = hidden, intermediate, float(limit), float(alpha)
+        self.gate_name, self.up_name, self.down_name = prefix + gate, prefix + up, prefix + down
+        self.w_gate_up = self.w_down = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, i = self.hidden, self.intermediate
+        return {self.gate_name: WeightSpec((i, h)), self.up_name: WeightSpec((i, h)), self.down_name: WeightSpec((h, i))}
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.w_gate_up = runtime.weight([tensors[self.gate_name], tensors[self.up_name]])
+        self.w_down = runtime.weight(tensors[self.down_name])
+
+    def _activated(self, h):
+        rt = self.runtime
+        sums = rt.empty((h.shape[0], 2 * self.intermediate), torch.float32)
+        rt.ops.linear(h, self.w_gate_up, sums)
+        act = rt.empty((h.shape[0], self.intermediate))
+        rt.ops.glu_clamped(sums, act, self.limit, self.alpha)
+        return act
+
+    def forward_into(self, h, batch, out: torch.Tensor) -> None:
+        self.runtime.ops.linear(self._activated(h), self.w_down, out)
+
+    def forward(self, h, batch, residual: torch.Tensor) -> None:
+        self.runtime.ops.linear(self._activated(h), self.w_down, residual, accumulate=True)
+
+
+class ExpertsMLP(FeedForward):
+    """A mixture of small gated feed-forwards (`e<n>.gate|up|down`, silu, no biases) of which every token uses `top`.
+    The router (`router` [experts, hidden]) gives logits in float32; scores are their sigmoids. Experts stand in
+    `groups` equal groups of neighbours, a group's score is the sum of its two largest scores, only experts of the `keep`
+    best groups can be chosen (groups None: all can); the `top` largest scores are chosen and divided by their sum
+    (+ 1e-20) as weights; the output is the weighted sum of the chosen experts' outputs.
+
+    Every expert's gate and up rows lie in one matrix and their down columns in another. A step of many tokens
+    multiplies every token with every expert, weights each expert's stretch of the activations by the router's weight (zero
+    for experts not chosen) and lets the down product add them up: two products of full tiles whatever the choice is, and a
+    token's result never depends on what else the step holds."""
+    capturable = True
+    GROUP_TOP = 2
+    WEIGHT_FLOOR = 1e-20
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, experts: int, top: int, groups=None, keep=None,
+                 router: str = "router", expert: str = "e{}.", gate: str = "gate", up: str = "up", down: str = "down"):
+        if experts <= 0 or not 0 < top <= experts:
+            raise ValueError(f"{top} of {experts} experts")
+        self.hidden, self.intermediate, self.experts, self.top = hidden, intermediate, int(experts), int(top)
+        self.groups, self.keep = (1, 1) if groups is None else (int(groups), int(keep))
+        if self.experts % self.groups != 0 or not 0 < self.keep <= self.groups or self.top > self.keep * (self.experts // self.groups):
+            raise ValueError(f"{experts} experts in {self.groups} groups, {self.keep} kept, {top} chosen")
+        self.router_name = prefix + router
+        self.expert_names = [tuple(prefix + expert.format(n) + name for name in (gate, up, down)) for n in range(self.experts)]
+        self.w_router = self.w_gate_up = self.w_down = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, i = self.hidden, self.intermediate
+        specs = {self.router_name: WeightSpec((self.experts, h))}
+        for gate, up, down in self.expert_names:
+            specs.update({gate: WeightSpec((i, h)), up: WeightSpec((i, h)), down: WeightSpec((h, i))})
+        return specs
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.w_router = runtime.matrix(tensors[self.router_name])
+        total = self.experts * self.intermediate
+        # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]
+        self.w_gate_up = runtime.weight([tensors[names[0]] for names in self.expert_names] + [tensors[names[1]] for names in self.expert_names],
+                                        "gated", gated_n=total)
+        down = torch.empty((self.hidden, total), dtype=runtime.dtype, device=runtime.device)
+        for n, names in enumerate(self.expert_names):
+            down[:, n * self.intermediate:(n + 1) * self.intermediate].copy_(tensors[names[2]])
+        self.w_down = runtime.weight(down)
+
+    def _weights(self, h):
+        rt = self.runtime
+        logits = rt.empty((h.shape[0], self.experts), torch.float32)
+        rt.ops.linear(h, self.w_router, logits)
+        weights = rt.empty((h.shape[0], self.experts), torch.float32)
+        rt.ops.route_experts(logits, weights, self.top, self.groups, self.keep, self.GROUP_TOP, self.WEIGHT_FLOOR)
+        return weights
+
+    def forward_into(self, h, batch, out: torch.Tensor) -> None:
+        rt = self.runtime
+        weights = self._weights(h)
+        act = rt.empty((h.shape[0], self.experts * self.intermediate))
+        rt.ops.linear_glu(h, self.w_gate_up, act, activation="silu")
+        rt.ops.scale_blocks(act, weights, self.intermediate)
+        rt.ops.linear(act, self.w_down, out)
+
+    def forward(self, h, batch, residual: torch.Tensor) -> None:
+        out = self.runtime.empty(residual.shape, torch.float32)
+        self.forward_into(h, batch, out)
+        self.runtime.ops.add(residual, out)
+
+
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "clamped_glu", ClampedGLU)
+register_part("feed_forward", "experts_mlp", ExpertsMLP)
 register_part("feed_forward", "dense_mlp", DenseMLP)

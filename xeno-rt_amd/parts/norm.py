@@ -102,6 +102,23 @@ class ScalarRMSNorm(RMSNorm):
         self.weight = runtime.vector(tensors[self.name]).reshape(1).expand(self.dim).contiguous()
 
 
+class OffsetRMSNorm(RMSNorm):
+    """RMSNorm whose tensor w holds the gain minus one: y = x / sqrt(mean(x^2) + eps) * (1 + w). `name` is the tensor that holds
+    w; 1 + w is worked out in float32 when the part is bound, and the norm then runs as any other."""
+
+    def __init__(self, name: str, dim: int, eps: float):
+        super().__init__(name, dim, eps)
+        self.name = name
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {self.name: WeightSpec((self.dim,), init="zeros", kind="vector")}
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        Norm.bind(self, tensors, runtime)
+        self.weight = (tensors[self.name].to(torch.float32) + 1.0).to(runtime.device).contiguous()
+
+
+register_part("norm", "offset_rmsnorm", OffsetRMSNorm)
 register_part("norm", "rmsnorm", RMSNorm)
 register_part("norm", "layernorm", LayerNorm)
 register_part("norm", "scalar_rmsnorm", ScalarRMSNorm)

@@ -95,12 +95,18 @@ class PairRotation(PositionEncoding):
     MAGNITUDE_SLOPE = 0.1
 
     def __init__(self, rope_dim: int, base: float, neighbours: bool = True, scaling: Optional[dict] = None):
+        """A second rule of stretching, by wavelength, is asked for with scaling = {factor, low, high, original}: with the
+        wavelength l = 2 pi / f a frequency stays where l < original / high, becomes f / factor where l > original / low, and
+        between the two, with s = (original / l - low) / (high - low), (1 - s) f / factor + s f; cosines and sines stay as
+        they are."""
         if rope_dim <= 0 or rope_dim % 2 != 0:
             raise ValueError(f"rotary width must be positive and even, found {rope_dim}")
         self.rope_dim, self.base, self.neighbours = int(rope_dim), float(base), bool(neighbours)
-        self.scaling = None if not scaling else {key: float(scaling[key]) for key in ("factor", "original", "fast", "slow")}
+        self.by_wavelength = bool(scaling) and "low" in scaling
+        keys = ("factor", "original", "low", "high") if self.by_wavelength else ("factor", "original", "fast", "slow")
+        self.scaling = None if not scaling else {key: float(scaling[key]) for key in keys}
         self.frequencies = None
-        self.magnitude = 1.0 if self.scaling is None else self.MAGNITUDE_SLOPE * math.log(self.scaling["factor"]) + 1.0
+        self.magnitude = 1.0 if self.scaling is None or self.by_wavelength else self.MAGNITUDE_SLOPE * math.log(self.scaling["factor"]) + 1.0
 
     def frequency_table(self):
         """The pairs' frequencies, as Python floats."""
@@ -108,6 +114,17 @@ class PairRotation(PositionEncoding):
         if self.scaling is None:
             return plain
         c = self.scaling
+        if self.by_wavelength:
+            out = []
+            for f in plain:
+                wavelength = 2.0 * math.pi / f
+                if wavelength > c["original"] / c["low"]:
+                    f = f / c["factor"]
+                elif wavelength >= c["original"] / c["high"]:
+                    share = (c["original"] / wavelength - c["low"]) / (c["high"] - c["low"])
+                    f = (1.0 - share) * f / c["factor"] + share * f
+                out.append(f)
+            return out
 
         def pair_of(turns: float) -> float:
             return self.rope_dim * math.log(c["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
