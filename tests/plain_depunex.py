@@ -5,7 +5,10 @@ x is the residual stream [tokens, width], h what a sublayer reads, t a token's i
 """
 from __future__ import annotations
 
+import json
 import math
+import os
+import struct
 
 import torch
 
@@ -42,10 +45,12 @@ def bigram_rows(tokens, buckets, mul_prev, mul_cur):
     return rows
 
 
-def embedding(tokens, table, bigram, scale, buckets, mul_prev, mul_cur):
+def embedding(tokens, table, scale, bigram=None, buckets=0, mul_prev=0, mul_cur=0):
     ids = torch.tensor(list(tokens), dtype=torch.long)
-    rows = torch.tensor(bigram_rows(list(tokens), buckets, mul_prev, mul_cur), dtype=torch.long)
-    return table.to(F)[ids] * scale + bigram.to(F)[rows]
+    x = table.to(F)[ids] * scale
+    if bigram is not None:
+        x = x + bigram.to(F)[torch.tensor(bigram_rows(list(tokens), buckets, mul_prev, mul_cur), dtype=torch.long)]
+    return x
 
 
 # ---- short causal convolution with bias, then silu ----------------------------------------------------------------------
@@ -148,9 +153,11 @@ def chunked_attention(h, p, m):
     if rot is not None:
         frequencies = rotary_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
         q, k = rotate(q, rot["dims"], frequencies), rotate(k, rot["dims"], frequencies)
-    size = m["mask"]["size"]
     i = torch.arange(tokens)
-    visible = (i[None, :] <= i[:, None]) & ((i[None, :] // size) == (i[:, None] // size))
+    visible = i[None, :] <= i[:, None]
+    if m.get("mask") is not None:
+        size = m["mask"]["size"]
+        visible = visible & ((i[None, :] // size) == (i[:, None] // size))
     out = torch.zeros(tokens, heads, vdim, dtype=F)
     for head in range(heads):
         shared = head // (heads // kv_heads)
@@ -175,8 +182,8 @@ def dense_ff(h, p, mlp):
     return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ p["down"].to(F).T
 
 
-def route(h, router, experts, top, group_count, group_keep):
-    """(chosen experts [tokens, top], their weights [tokens, top])."""
+def route(h, router, experts, top, group_count=1, group_keep=1):
+    """(chosen experts [tokens, top], their weights [tokens, top]). One group: every expert can be chosen."""
     scores = torch.sigmoid(h @ router.to(F).T)                                # [tokens, experts]
     tokens = h.shape[0]
     per_group = experts // group_count
@@ -194,7 +201,8 @@ def route(h, router, experts, top, group_count, group_keep):
 
 def moe_ff(h, p, mlp):
     r = mlp["router"]
-    chosen, weights = route(h, p["router"], r["experts"], r["top"], r["groups"]["count"], r["groups"]["keep"])
+    groups = r.get("groups") or {"count": 1, "keep": 1}
+    chosen, weights = route(h, p["router"], r["experts"], r["top"], groups["count"], groups["keep"])
     out = torch.zeros(h.shape[0], p["e0.down"].shape[0], dtype=F)
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t].tolist(), weights[t]):
@@ -238,9 +246,12 @@ def layer_forward(x, tokens, index, layer, tensors, config):
 
 def forward(tokens, tensors, config, streams=None):
     """Logits [tokens, vocab] of one whole sequence; `streams`, a list, receives the residual stream after every layer."""
-    e = config["embedding"]
-    b = e["bigram"]
-    x = embedding(tokens, tensors["embed"], tensors["bigram"], e["scale"], b["buckets"], b["mul_prev"], b["mul_cur"])
+    e = config.get("embedding") or {}
+    b = e.get("bigram")
+    if b is None:
+        x = embedding(tokens, tensors["embed"], e.get("scale", 1.0))
+    else:
+        x = embedding(tokens, tensors["embed"], e.get("scale", 1.0), tensors["bigram"], b["buckets"], b["mul_prev"], b["mul_cur"])
     for index, layer in enumerate(config["layers"]):
         x = layer_forward(x, tokens, index, layer, tensors, config)
         if streams is not None:
@@ -249,3 +260,39 @@ def forward(tokens, tensors, config, streams=None):
     logits = y @ tensors["embed"].to(F).T
     cap = config.get("logit_softcap")
     return logits if cap is None else cap * torch.tanh(logits / cap)
+
+
+
+def read_folder(folder):
+    """(config.json as a dict, {name: tensor as stored}) of a model folder; the file's layout is read here, by hand."""
+    with open(os.path.join(folder, "config.json")) as handle:
+        raw = json.load(handle)
+    with open(os.path.join(folder, "model.safetensors"), "rb") as handle:
+        size = struct.unpack("<Q", handle.read(8))[0]
+        header = json.loads(handle.read(size))
+        data = handle.read()
+    kinds = {"BF16": torch.bfloat16, "F32": torch.float32, "F16": torch.float16, "I32": torch.int32}
+    tensors = {}
+    for name, entry in header.items():
+        if name != "__metadata__":
+            lo, hi = entry["data_offsets"]
+            tensors[name] = torch.frombuffer(bytearray(data[lo:hi]), dtype=kinds[entry["dtype"]]).reshape(entry["shape"])
+    return raw, tensors
+
+
+class PlainModel:
+    def __init__(self, folder):
+        self.raw, self.tensors = read_folder(folder)
+
+    def logits(self, tokens):
+        with torch.no_grad():
+            return forward(list(tokens), self.tensors, self.raw).to(torch.float32)
+
+
+def generate_greedy(model, prompt, count):
+    ids, out = list(prompt), []
+    for _ in range(count):
+        token = int(model.logits(ids)[-1].argmax())
+        out.append(token)
+        ids.append(token)
+    return out

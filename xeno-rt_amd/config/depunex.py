@@ -153,7 +153,10 @@ class DepunexConfig:
         if bigram is not None:
             if not isinstance(bigram, dict):
                 raise ConfigError("config.json: 'embedding.bigram' must be an object")
-            _sizes(bigram, ("buckets", "mul_prev", "mul_cur"), "embedding.bigram")
+            _sizes(bigram, ("buckets",), "embedding.bigram")
+            for key in ("mul_prev", "mul_cur"):
+                if isinstance(bigram.get(key), bool) or not isinstance(bigram.get(key), int) or not 0 <= bigram[key] < 2 ** 31:
+                    raise ConfigError(f"config.json: embedding.bigram: '{key}' must be an integer from 0 up, found {bigram.get(key)!r}")
             bigram = (int(bigram["buckets"]), int(bigram["mul_prev"]), int(bigram["mul_cur"]))
         side = raw.get("token_side")
         if side is not None:

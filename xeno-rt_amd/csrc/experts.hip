@@ -87,7 +87,7 @@ extern "C" int xrt_route_experts(const float* logits, long tokens, int experts, 
                                  float* weights, int* chosen, void* stream) {
     XRT_REQUIRE(logits && weights && tokens >= 0, "route_experts: null operand");
     XRT_REQUIRE(experts > 0 && experts <= XRT_MOST_EXPERTS && top > 0 && groups > 0 && experts % groups == 0 && keep > 0 && keep <= groups &&
-                group_top > 0 && experts / groups <= 128 && top <= keep * (experts / groups),
+                group_top > 0 && (groups == 1 || experts / groups <= 128) && top <= keep * (experts / groups),
                 "route_experts: %d experts in %d groups of which %d are kept, %d chosen: up to %d experts in equal groups, and no more "
                 "chosen than the kept groups hold", experts, groups, keep, top, XRT_MOST_EXPERTS);
     if (tokens == 0) return 0;

@@ -122,7 +122,7 @@ class SandwichBlock(Block):
         return specs
 
     def ignored_names(self):
-        return self.unread + [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
+        return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
 
     def cache_needs(self) -> CacheNeeds:
         return self.mixer.cache_needs().merged(*([self.mixer_input.cache_needs()] if self.mixer_input is not None else []))
