@@ -30,6 +30,13 @@ tokens a second and ms; one JSON line with both models' numbers.
 the same for the Ledudra decoder (attention with sigmoid weights, mixed heads and a gate under a window of 512 keys, and
 softmax attention with head norms and biases by distance under a window of 1024, in turn, every sublayer between two
 layer norms), beside the same Llama decoder.
+
+    python bench.py --design depunex [--size small|medium|large] [--layers N]
+
+the same for the Depunex decoder (layers of a matrix state per head with step sizes, and of attention inside chunks of 512
+positions beside a selective scan, in turn; a clamped gated feed-forward or eight experts of which a token uses two, in
+turn; the hashed table of token pairs, the per-layer side input and the capped logits), beside the Sozopel decoder, the
+library's closest (recurrences, short convolutions, two mixers side by side on the general attention kernel), and Llama.
 """
 import argparse
 import json
@@ -142,7 +149,24 @@ def ledudra_config(size, layers, max_positions):
             "layers": [kinds[i % 2] for i in range(layers)]}
 
 
-DESIGN_CONFIGS = {"sozopel": sozopel_config, "ledudra": ledudra_config}
+def depunex_config(size, layers, max_positions):
+    w, d, ff = size["width"], size["head"], size["ff"]
+    heads = w // d
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    experts = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    duality = {"heads": 2 * heads, "vdim": d, "state": 128, "groups": 1, "norm_groups": 1, "conv": 4}
+    pair = {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": d, "vdim": d, "mask": {"size": 512}, "scale": d ** -0.5,
+                     "rot": {"dims": d // 2, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}}},
+            "right": {"inner": w, "state": 16, "dt_rank": max(1, w // 16), "conv": 4}, "left_scale": 0.5, "right_scale": 0.5}
+    kinds = [{"type": "mamba2", "mixer": duality, "mlp": dense}, {"type": "parallel", "mixer": pair, "mlp": experts},
+             {"type": "mamba2", "mixer": duality, "mlp": experts}, {"type": "parallel", "mixer": pair, "mlp": dense}]
+    return {"architecture": "Depunex", "vocab": size["vocab"], "width": w, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "embedding": {"scale": w ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "token_side": {"dim": 64},
+            "layers": [kinds[i % 4] for i in range(layers)]}
+
+
+DESIGN_CONFIGS = {"sozopel": sozopel_config, "ledudra": ledudra_config, "depunex": depunex_config}
+DESIGN_BESIDE = {"depunex": ("sozopel", "llama")}          # the models a design is measured beside (Llama alone unless named)
 
 
 def llama_config(size, layers, max_positions):
@@ -159,9 +183,11 @@ def run_design(args) -> int:
     layers = args.layers if args.layers is not None else 6
     context = DESIGN_CONTEXT
     most = max(DESIGN_BATCHES)
-    record = {"design": args.design, "beside": "llama", "size": args.size, **size, "layers": layers, "dtype": args.dtype,
+    beside = DESIGN_BESIDE.get(args.design, ("llama",))
+    record = {"design": args.design, "beside": ", ".join(beside), "size": args.size, **size, "layers": layers, "dtype": args.dtype,
               "context": context, "prefill_tokens": PREFILL_TOKENS, "data": "synthetic token ids, random weights N(0, 0.02)"}
-    for name, raw in ((args.design, DESIGN_CONFIGS[args.design](size, layers, 4096)), ("llama", llama_config(size, layers, 4096))):
+    configs = {**DESIGN_CONFIGS, "llama": llama_config}
+    for name, raw in [(name, configs[name](size, layers, 4096)) for name in (args.design, *beside)]:
         engine = Engine.random(parse_config(raw), seed=args.seed, dtype=args.dtype, max_tokens=max(most * context, PREFILL_TOKENS),
                                max_slots=most, max_context=max(context, PREFILL_TOKENS))
         bench = Bench(engine, args.seed)
