@@ -394,15 +394,17 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_r
 
 // The same for a norm that comes after the gate and spans equal parts of the token's whole row (heads x vdim), whatever the
 // heads are: value = raw (+ skip * v) times the gate, then divided by the root mean square of its part, times the weight
-// [heads * vdim]. A workgroup per (token, part).
-__global__ void __launch_bounds__(256) recurrence_finish_groups_kernel(const xrt_recurrence a, int dtype, const float* __restrict__ raw,
-                                                                      const int* __restrict__ token_slots, int row_split, long tokens) {
+// [heads * vdim]. A workgroup per (token, part); a thread keeps up to FINISH_KEPT of its gated values in registers between the
+// pass that sums their squares and the pass that writes them (columns beyond that are worked out twice).
+constexpr int FINISH_THREADS = 512, FINISH_KEPT = 8;
+__global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kernel(const xrt_recurrence a, int dtype, const float* __restrict__ raw,
+                                                                                 const int* __restrict__ token_slots, int row_split, long tokens) {
     __shared__ float scratch[32];
     const long row = blockIdx.x;
     const int width = a.heads * a.vdim, part_width = width / a.norm_groups, c0 = blockIdx.y * part_width;
     const long out_at = row * width;
     if (token_slots[row] < 0) {
-        for (int c = threadIdx.x; c < part_width; c += blockDim.x) store_from_float(a.out, dtype, out_at + c0 + c, 0.f);
+        for (int c = threadIdx.x; c < part_width; c += FINISH_THREADS) store_from_float(a.out, dtype, out_at + c0 + c, 0.f);
         return;
     }
     auto gated = [&](int c) {                              // c: a column of the whole row
@@ -415,10 +417,26 @@ __global__ void __launch_bounds__(256) recurrence_finish_groups_kernel(const xrt
         }
         return sum;
     };
+    float kept[FINISH_KEPT];
     float squares = 0.f;
-    for (int c = threadIdx.x; c < part_width; c += blockDim.x) { const float o = gated(c0 + c); squares = fmaf(o, o, squares); }
+#pragma unroll
+    for (int i = 0; i < FINISH_KEPT; ++i) {
+        const int c = threadIdx.x + i * FINISH_THREADS;
+        kept[i] = c < part_width ? gated(c0 + c) : 0.f;
+        squares = fmaf(kept[i], kept[i], squares);
+    }
+    for (int c = threadIdx.x + FINISH_KEPT * FINISH_THREADS; c < part_width; c += FINISH_THREADS) { const float o = gated(c0 + c); squares = fmaf(o, o, squares); }
     const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)part_width + a.eps);
-    for (int c = threadIdx.x; c < part_width; c += blockDim.x) {
+#pragma unroll
+    for (int i = 0; i < FINISH_KEPT; ++i) {
+        const int c = threadIdx.x + i * FINISH_THREADS;
+        if (c < part_width) {
+            float value = kept[i] * inv;
+            if (a.norm_weight != nullptr) value *= load_as_float(a.norm_weight, a.norm_weight_dtype, c0 + c);
+            store_from_float(a.out, dtype, out_at + c0 + c, value);
+        }
+    }
+    for (int c = threadIdx.x + FINISH_KEPT * FINISH_THREADS; c < part_width; c += FINISH_THREADS) {
         float value = gated(c0 + c) * inv;
         if (a.norm_weight != nullptr) value *= load_as_float(a.norm_weight, a.norm_weight_dtype, c0 + c);
         store_from_float(a.out, dtype, out_at + c0 + c, value);
@@ -598,7 +616,7 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
 #undef XRT_REC_DIM
 #undef XRT_REC
     if (a.norm_groups > 0)
-        recurrence_finish_groups_kernel<<<dim3((unsigned)tokens, a.norm_groups), 256, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
+        recurrence_finish_groups_kernel<<<dim3((unsigned)tokens, a.norm_groups), FINISH_THREADS, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
     else
         recurrence_finish_kernel<<<dim3((unsigned)tokens, a.heads), XRT_WAVE, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
     XRT_LAUNCH_CHECK("linear_recurrence");

@@ -2,7 +2,8 @@
 //   xrt_bigram_add      x <- x * scale + table[row], the row hashed from the token and the one before it; the token before a
 //                       step's first is kept per sequence
 //   xrt_gated_rows      out[t][c] = gelu_tanh(s[t][c]) * table[ids[t]][offset + c]: a slice of a token's row of a table, gated
-//   xrt_add_weighted    residual += sum of scale_n * gain_n * y_n over up to four float32 matrices (gains per column, or none)
+//   xrt_add_weighted    residual += sum of scale_n * gain_n * y_n over up to four float32 matrices (gains per column, or none);
+//                       the updated rows may be written once more in another element type, for a product that reads them
 //   xrt_glu_clamped     out = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit), from
 //                       float32 sums [rows][2 n] that hold g then u
 //   xrt_softcap         x <- cap * tanh(x / cap), in place on float32
@@ -77,7 +78,7 @@ struct WeightedTerms {
     int count, gain_dtype;
 };
 
-__global__ void add_weighted_kernel(float* __restrict__ residual, WeightedTerms terms, long count, int width) {
+__global__ void add_weighted_kernel(float* __restrict__ residual, WeightedTerms terms, long count, int width, void* __restrict__ copy, int copy_dtype) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= count) return;
     const int c = (int)(i % width);
@@ -90,7 +91,9 @@ __global__ void add_weighted_kernel(float* __restrict__ residual, WeightedTerms 
             sum += v;
         }
     }
-    residual[i] += sum;
+    const float updated = residual[i] + sum;
+    residual[i] = updated;
+    if (copy != nullptr) store_from_float(copy, copy_dtype, i, updated);
 }
 
 __global__ void glu_clamped_kernel(const float* __restrict__ sums, void* __restrict__ out, int out_dtype, long rows, int n, float limit, float alpha) {
@@ -147,7 +150,8 @@ extern "C" int xrt_gated_rows(const float* s, long s_stride, const void* table, 
 }
 
 extern "C" int xrt_add_weighted(float* residual, int count, const float* const* y, const void* const* gains, const float* scales, int gain_dtype,
-                                long rows, int width, void* stream) {
+                                long rows, int width, void* copy, int copy_dtype, void* stream) {
+    XRT_REQUIRE(copy == nullptr || known(copy_dtype), "add_weighted: unknown dtype of the copy");
     XRT_REQUIRE(residual && y && gains && scales && count >= 1 && count <= 4 && known(gain_dtype), "add_weighted: one to four terms");
     XRT_REQUIRE(rows >= 0 && width > 0, "add_weighted: bad sizes");
     if (rows == 0) return 0;
@@ -162,7 +166,7 @@ extern "C" int xrt_add_weighted(float* residual, int count, const float* const* 
     }
     const long blocks = (rows * width + 255) / 256;
     XRT_REQUIRE(blocks < (1L << 31), "add_weighted: too many elements");
-    add_weighted_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(residual, terms, rows * width, width);
+    add_weighted_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(residual, terms, rows * width, width, copy, copy_dtype);
     XRT_LAUNCH_CHECK("add_weighted");
     return 0;
 }

@@ -366,9 +366,10 @@ int xrt_bigram_add(float* x, long tokens, int width, float scale, const void* ta
 // out[t][c] = gelu_tanh(s[t][c]) * table[ids[t]][offset + c] for c < width; s float32 rows s_stride apart; table [rows][table_width]
 int xrt_gated_rows(const float* s, long s_stride, const void* table, int table_dtype, long table_width, long offset, int rows,
                    const int* ids, void* out, int out_dtype, long tokens, int width, void* stream);
-// residual += sum over n < count of scales[n] * gains[n][column] * y[n] (y float32 [rows][width]; a null gain is all ones)
+// residual += sum over n < count of scales[n] * gains[n][column] * y[n] (y float32 [rows][width]; a null gain is all ones);
+// copy (or null): the updated rows once more, in copy_dtype
 int xrt_add_weighted(float* residual, int count, const float* const* y, const void* const* gains, const float* scales, int gain_dtype,
-                     long rows, int width, void* stream);
+                     long rows, int width, void* copy, int copy_dtype, void* stream);
 // out[r][c] = g * sigmoid(alpha * g) * (u + 1), g = min(sums[r][c], limit), u = clamp(sums[r][n + c], -limit, limit)
 int xrt_glu_clamped(const float* sums, void* out, int out_dtype, long rows, int n, float limit, float alpha, void* stream);
 // x <- cap * tanh(x / cap), float32 in place

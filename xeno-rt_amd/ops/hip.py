@@ -888,9 +888,9 @@ class HipOps:
                                             ctypes.c_long(offset), table.shape[0], _ptr(ids), _ptr(out), _code(out), ctypes.c_long(tokens),
                                             width, self._stream(s)))
 
-    def add_weighted(self, residual, terms):
+    def add_weighted(self, residual, terms, copy=None):
         """residual += sum over (y, gain, scale) in terms of scale * gain * y; y float32 like residual, gain [width] or None; one to
-        four terms."""
+        four terms. copy: a tensor shaped like residual that takes the updated rows in its own element type."""
         self._require(residual, "add_weighted residual", torch.float32)
         if residual.dim() != 2 or not 1 <= len(terms) <= 4:
             raise KernelError("add_weighted: a residual [rows, width] and one to four terms")
@@ -904,8 +904,10 @@ class HipOps:
         ys = (ctypes.c_void_p * count)(*[y.data_ptr() for y, _, _ in terms])
         gs = (ctypes.c_void_p * count)(*[0 if gain is None else gain.data_ptr() for _, gain, _ in terms])
         scales = (ctypes.c_float * count)(*[float(scale) for _, _, scale in terms])
+        if copy is not None:
+            self._require(copy, "add_weighted copy", None, (rows, width), residual)
         self._check(self.lib.xrt_add_weighted(_ptr(residual), count, ys, gs, scales, _code(gains[0]) if gains else 0, ctypes.c_long(rows),
-                                              width, self._stream(residual)))
+                                              width, _ptr(copy), 0 if copy is None else _code(copy), self._stream(residual)))
 
     def glu_clamped(self, sums, out, limit, alpha):
         """out = g * sigmoid(alpha g) * (u + 1) with g = min(sums[:, :n], limit), u = clamp(sums[:, n:], -limit, limit)."""

@@ -160,7 +160,8 @@ class ParallelBlock(Block):
     are vectors over the model width (`mixer_scale`, `feed_forward_scale`: tensor names, or None for ones). The sublayers
     write their float32 outputs aside and one pass adds them to the stream; a mixer that is itself a weighted sum of
     mixers (`forward_terms`) has its terms added in that same pass. `after`, if given, is a part that then adds what the
-    step's tokens bring to the stream of their own (`forward(x, batch)`)."""
+    step's tokens bring to the stream of their own (`forward(x, batch, reads=)`, reads being x in the compute dtype if the
+    block has it at hand)."""
 
     def __init__(self, norm, mixer, feed_forward=None, hidden=None, mixer_scale=None, feed_forward_scale=None, after=None):
         self.norm, self.mixer, self.feed_forward, self.after = norm, mixer, feed_forward, after
@@ -212,9 +213,11 @@ class ParallelBlock(Block):
             y = rt.empty(x.shape, torch.float32)
             self.feed_forward.forward_into(h, batch, y)
             terms.append((y, self.scales[1], 1.0))
-        rt.ops.add_weighted(x, terms)
+        # what follows reads the updated stream in the compute dtype: written in the same pass
+        reads = rt.empty(x.shape) if self.after is not None and rt.dtype != torch.float32 else None
+        rt.ops.add_weighted(x, terms, copy=reads)
         if self.after is not None:
-            self.after.forward(x, batch)
+            self.after.forward(x, batch, reads=reads)
 
 
 register_part("block", "parallel", ParallelBlock)

@@ -156,13 +156,15 @@ class TokenSideInput(Part):
         self.w_proj = runtime.weight(tensors[self.proj_name])
         self.norm_weight = runtime.vector(tensors[self.norm_name])
 
-    def forward(self, x: torch.Tensor, batch) -> None:
+    def forward(self, x: torch.Tensor, batch, reads=None) -> None:
+        """reads: x in the compute dtype, if the caller has it already."""
         rt = self.runtime
         tokens, dim = x.shape[0], self.side.dim
-        reads = x
-        if rt.dtype != torch.float32:
-            reads = rt.empty(x.shape)
-            rt.ops.cast(x, reads)
+        if reads is None:
+            reads = x
+            if rt.dtype != torch.float32:
+                reads = rt.empty(x.shape)
+                rt.ops.cast(x, reads)
         sums = rt.empty((tokens, dim), torch.float32)
         rt.ops.linear(reads, self.w_gate, sums)
         g = rt.empty((tokens, dim))
