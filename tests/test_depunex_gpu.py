@@ -447,10 +447,44 @@ def test_attention_inside_chunks_of_positions(n_heads, n_kv_heads, dim, vdim, ch
         got = attend(ops, q, k, v, cuts, dtype, n_heads, n_kv_heads, dim, vdim, scale=scale, chunk=chunk)
         limit = 1e-5 if dtype == torch.float32 else 2e-2
         assert float((got - want).abs().max()) <= limit * float(want.abs().max()), f"chunk {chunk}, cuts {cuts[:4]}"
+        # (bfloat16 heads of 64 or 128 dims in chunks of whole cache blocks: steps of several tokens go to the matrix cores,
+        # steps of one token do not, and the two agree but for rounding)
         if first is None:
             first = got
-        else:
+        elif not (dtype == torch.bfloat16 and dim == vdim and dim in (64, 128) and (chunk or 0) % 64 == 0):
             assert torch.equal(got, first), f"cuts {cuts[:4]} change the bits"
+
+
+@pytest.mark.parametrize("n_heads,n_kv_heads,dim,chunk", [(4, 2, 64, 64), (2, 1, 128, 128), (4, 4, 128, 192), (6, 2, 64, 320), (2, 2, 128, None),
+                                                          (8, 2, 128, 512)])
+def test_attention_inside_chunks_on_the_matrix_cores(n_heads, n_kv_heads, dim, chunk, ops):
+    """Prompts long enough for several tiles of queries in one chunk, whole and in portions that begin and end inside chunks,
+    on chunk borders and on cache block borders, against the plain sum; the probabilities keep sixteen bits, so the error
+    is that of the rounded operands and result."""
+    length = 700
+    generator = torch.Generator().manual_seed(dim + n_heads)
+    q, k = torch.randn(length, n_heads * dim, generator=generator), torch.randn(length, n_kv_heads * dim, generator=generator)
+    v = torch.randn(length, n_kv_heads * dim, generator=generator)
+    q, k, v = (t.to(torch.bfloat16).float() for t in (q, k, v))
+    scale = 1.5 / math.sqrt(dim)
+    want = plain_chunked(q, k, v, n_heads, n_kv_heads, dim, dim, scale, chunk)
+    for cuts in ([length], [length - 3, 1, 2], [70, length - 70], [64, 64, 300, 272], [129, 257, 2, 312], [5] * 140, [191, 193, 316]):
+        got = attend(ops, q, k, v, cuts, torch.bfloat16, n_heads, n_kv_heads, dim, dim, scale=scale, chunk=chunk)
+        error = (got - want).abs()
+        assert float(error.max()) <= 6e-3 * float(want.abs().max()), f"chunk {chunk}, cuts {cuts[:4]}: row {int(error.max(dim=1).values.argmax())}"
+
+
+@pytest.mark.parametrize("chunk", [64, 128, 192])
+def test_the_matrix_cores_see_a_chunks_first_key_and_not_the_one_before(chunk, ops):
+    n_heads, dim, length = 2, 64, 450
+    for query in sorted({chunk, 2 * chunk - 1, chunk + chunk // 2, (449 // chunk) * chunk, 449}):
+        first = query - query % chunk
+        for key, seen in ((first, True), (first - 1, False)):
+            q, k, v = (torch.zeros(length, n_heads * dim) for _ in range(3))
+            q[query], k[key], v[key] = 3.0, 3.0, 1.0
+            for cuts in ([length], [query - 1, 2, length - query - 1], [first, length - first], [first + 1, length - first - 1]):
+                got = attend(ops, q, k, v, cuts, torch.bfloat16, n_heads, n_heads, dim, dim, scale=0.05, chunk=chunk)
+                assert abs(float(got[query, 0]) - (1.0 if seen else 0.0)) < 1e-2, f"chunk {chunk}, query {query}, key {key}, cuts {cuts}"
 
 
 @pytest.mark.parametrize("chunk", [1, 3, 20, 64, 70, 128])

@@ -17,10 +17,10 @@ int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_head
                          const int* positions, const int* slots, void* out, float scale, int max_context,
                          float* workspace, long workspace_floats, const xrt_qkv_finish* finish, hipStream_t s);
 bool xrt_attention_prefill_accepts(int head_dim);
-int xrt_attention_prefill(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
+int xrt_attention_prefill(const void* qkv, long q_stride, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                           const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
-                          float scale, hipStream_t s);
+                          float scale, int stretch, bool fine, hipStream_t s);
 
 static bool takes_decode_kernel(int dtype, int n_heads, int n_kv_heads, int head_dim, int window, int max_count, int max_context) {
     return dtype == XRT_BF16 && window == 0 && max_count == 1 && max_context > 0 && n_heads > 0 && n_kv_heads > 0 &&
@@ -60,9 +60,9 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
             // tokens beyond the sequences (padding) get zeros
             // (their rows are read by nothing, but must not hold what a later product could choke on)
             XRT_REQUIRE(n_seqs <= tokens, "attention: more sequences than tokens");
-            return xrt_attention_prefill(qkv, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
+            return xrt_attention_prefill(qkv, 0, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
                                          table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, out,
-                                         scale, s);
+                                         scale, 0, false, s);
         }
     }
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, head_dim, k_cache, v_cache, block_table,
@@ -92,6 +92,28 @@ extern "C" int xrt_attention_general(const void* qkv, int dtype, int tokens, int
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, value_dim, k_cache, v_cache, block_table,
                                  table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, sink, q_stride,
                                  distance_bias, bias_span, chunk, (hipStream_t)stream);
+}
+
+// ---- the matrix-core kernel for a step of many tokens whose queries see their own stretch of positions only (xrt_hip.h)
+
+extern "C" int xrt_attention_stretches_accepts(int dtype, int head_dim, int value_dim, int chunk) {
+    return dtype == XRT_BF16 && head_dim == value_dim && xrt_attention_prefill_accepts(head_dim) && chunk >= 0 &&
+           chunk % XRT_BLOCK_TOKENS == 0;
+}
+
+extern "C" int xrt_attention_stretches(const void* q, long q_stride, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                                       const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                                       const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
+                                       float scale, int chunk, void* stream) {
+    XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+                "attention: head counts %d/%d: the first must be a multiple of the second", n_heads, n_kv_heads);
+    XRT_REQUIRE(xrt_attention_stretches_accepts(dtype, head_dim, head_dim, chunk),
+                "attention (stretches): bfloat16, heads of 64 or 128 dims and stretches of whole cache blocks only (found %d, %d)", head_dim, chunk);
+    XRT_REQUIRE(q && k_cache && v_cache && block_table && seq_offsets && seq_slots && seq_starts && out, "attention: null operand");
+    XRT_REQUIRE(table_stride > 0 && n_blocks > 0 && n_seqs > 0 && n_seqs <= tokens, "attention: empty cache, or no sequences");
+    if (tokens == 0) return 0;
+    return xrt_attention_prefill(q, q_stride, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table, table_stride, n_blocks,
+                                 seq_offsets, seq_slots, seq_starts, n_seqs, out, scale, chunk, true, (hipStream_t)stream);
 }
 
 // ---- a decode step whose attention also finishes q, k and v (xrt_hip.h)

@@ -20,6 +20,7 @@
 // product wants as its B operand: key rows are assigned to accumulator rows such that a lane
 // holds eight consecutive keys per K step, which are also 16 contiguous bytes of the
 // transposed value block.
+#include <climits>
 #include "cache_layout.h"
 #include "xrt_hip.h"
 
@@ -49,12 +50,14 @@ constexpr int GROUPS = 4;              // groups of 32 queries in a tile
 constexpr int WAVES = 2 * GROUPS;
 constexpr int QW = GROUPS * QT;        // queries of a tile
 
-template <int HD>
+// FINE: the probabilities enter the value product as two bfloat16 numbers each, the rounded one and what the rounding left
+// (sixteen bits of them instead of eight, for twice the value products), for models whose weights are float32.
+template <int HD, bool FINE>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ seq_offsets, const int* __restrict__ seq_slots,
-    const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale) {
+    const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale, int stretch) {
     constexpr int KS = HD / 16;            // K steps of the score product
     constexpr int DT = HD / 32;            // 32-row tiles of the value product
     constexpr int K_CHUNKS = HD / 8;       // 16-byte chunks of a key row (16 or 8)
@@ -80,18 +83,31 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     const int group = wave_uniform % GROUPS;                 // the 32 queries of a tile that this wavefront holds
     const bool helper = wave_uniform >= GROUPS;              // early tile first, then half of the late tile's blocks
 
-    // which sequence and which pair of its tiles this workgroup has
-    int pair = blockIdx.y, seq = 0, count = 0, tiles = 0;
+    // Which sequence and which pair of its tiles this workgroup has. With stretches of positions (stretch > 0, a multiple of
+    // the cache block: a query sees the keys of its own stretch only, stretches counted from the sequence's first token) every
+    // part of a sequence's new tokens that lies in one stretch is served like a sequence of its own, whose cache begins at
+    // the stretch's first block and whose positions count from the stretch's start.
+    int pair = blockIdx.y, seq = 0, count = 0, tiles = 0, start = 0, first_block = 0, first_token = 0;
+    bool found = false;
     for (; seq < n_seqs; ++seq) {
-        count = seq_offsets[seq + 1] - seq_offsets[seq];
-        tiles = (count + QW - 1) / QW;
-        const int pairs = (tiles + 1) / 2;
-        if (pair < pairs) break;
-        pair -= pairs;
+        const int whole = seq_offsets[seq + 1] - seq_offsets[seq], begin = seq_starts[seq];
+        for (int p = begin; p < begin + whole; p += count) {
+            count = stretch > 0 ? min(begin + whole, (p / stretch + 1) * stretch) - p : whole;
+            tiles = (count + QW - 1) / QW;
+            const int pairs = (tiles + 1) / 2;
+            if (pair < pairs) {
+                found = true;
+                first_token = seq_offsets[seq] + (p - begin);
+                start = stretch > 0 ? p % stretch : p;           // tokens in the cache (of the stretch) before these
+                first_block = stretch > 0 ? p / stretch * (stretch / BT) : 0;
+                break;
+            }
+            pair -= pairs;
+        }
+        if (found) break;
     }
-    if (seq >= n_seqs) return;                               // the whole workgroup leaves
+    if (!found) return;                                      // the whole workgroup leaves
     const int slot = seq_slots[seq];
-    const int start = seq_starts[seq];                       // tokens in the cache before this step
     const int late_tile = tiles - 1 - pair, early_tile = pair;
     const bool has_early = early_tile < late_tile;
     // blocks of keys that the two tiles see: the early tile 0 .. early_blocks - 1, the late tile 0 .. late_blocks - 1
@@ -111,7 +127,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         const int q_first = tile * QW + group * QT;
         q_count = max(0, min(QT, count - q_first));          // queries of this wavefront that exist
         q_valid = col < q_count;
-        token = (long)seq_offsets[seq] + min(q_first + col, count - 1);
+        token = (long)first_token + min(q_first + col, count - 1);
         q_pos = start + q_first + col;                       // absolute position of this lane's query
         last_key = q_count > 0 ? start + q_first + q_count - 1 : -1;     // the furthest key any query of the wavefront sees
         first_masked = start + q_first;                      // key tiles that end at or before this need no mask
@@ -164,8 +180,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     const unsigned lds_k0 = lds_address(lds_raw), lds_v0 = lds_k0 + 2 * PER_STAGE * BT * HD * (unsigned)sizeof(bf16);
     // The table's entries are read a stage before they are used: read where they are used, every stage would begin
     // with the wait for a scalar load.
-    const int* table = block_table + (long)slot * table_stride;
-    auto block_of = [&](int b) { return table[min(b, table_stride - 1)]; };
+    const int* table = block_table + (long)slot * table_stride + first_block;
+    auto block_of = [&](int b) { return table[min(b, table_stride - 1 - first_block)]; };
     auto fetch = [&](int block, int buffer) {
         block = min(max(block, 0), n_blocks - 1);            // the host never hands out anything else
         const char* kb = reinterpret_cast<const char*>(k_cache + ((long)block * n_kv_heads + kv_head) * BT * HD);
@@ -265,12 +281,14 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         }
         const float m_safe = m == -INFINITY ? 0.f : m;        // a query that sees none of these keys yet
 
-        bf16x8 p[2];
+        bf16x8 p[2], p_rest[FINE ? 2 : 1];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const float e = __builtin_amdgcn_exp2f(fmaf(s[i], scale2, -m_safe));
             l += e;
-            p[i / 8][i % 8] = (bf16)e;
+            const bf16 rounded = (bf16)e;
+            p[i / 8][i % 8] = rounded;
+            if constexpr (FINE) p_rest[i / 8][i % 8] = (bf16)(e - (float)rounded);
         }
 #pragma unroll
         for (int step = 0; step < 2; ++step) {
@@ -285,6 +303,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v[dt], p[step], o[dt], 0, 0, 0);
+                if constexpr (FINE) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v[dt], p_rest[step], o[dt], 0, 0, 0);
                 if (step == 0) v[dt] = v_at(1, dt);    // the values of the other 16 keys, behind the product that used the register
             }
         }
@@ -369,50 +388,50 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     write_out();
 }
 
-template <int HD>
-int launch_waves(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
+template <int HD, bool FINE>
+int launch_waves(const bf16* qkv, long q_stride, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
                  const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
-                 const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
-    const int row_width = (n_heads + 2 * n_kv_heads) * HD;
-    // a sequence of `count` tokens has ceil(ceil(count / QW) / 2) pairs of tiles; their sum is at most this
-    const long pairs = ((tokens + QW - 1) / QW + n_seqs) / 2 + n_seqs;
+                 const int* seq_starts, int n_seqs, bf16* out, float scale, int stretch, hipStream_t s) {
+    const int row_width = q_stride > 0 ? (int)q_stride : (n_heads + 2 * n_kv_heads) * HD;
+    // a run of `count` tokens has ceil(ceil(count / QW) / 2) pairs of tiles; their sum is at most this. A sequence is one run,
+    // or with stretches of positions a run per stretch that its new tokens touch.
+    const long runs = stretch > 0 ? tokens / stretch + 2L * n_seqs : n_seqs;
+    const long pairs = ((tokens + QW - 1) / QW + runs) / 2 + runs;
     XRT_REQUIRE(pairs <= 65535, "attention (prefill): too many query tiles for the grid");
     const dim3 grid(n_heads, (unsigned)pairs);
     constexpr size_t lds = (size_t)2 * PER_STAGE * (BT * HD + HD * BT) * sizeof(bf16);
     static_assert(lds >= GROUPS * (HD / 32 * 16 + 2) * XRT_WAVE * sizeof(float), "the merge does not fit the blocks' buffers");
     static bool configured = false;          // per instantiation
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD, FINE>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         XRT_REQUIRE(e == hipSuccess, "attention (prefill): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         configured = true;
     }
-    attention_prefill_kernel<HD><<<grid, WAVES * XRT_WAVE, lds, s>>>(
+    attention_prefill_kernel<HD, FINE><<<grid, WAVES * XRT_WAVE, lds, s>>>(
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, seq_offsets,
-        seq_slots, seq_starts, n_seqs, out, scale);
+        seq_slots, seq_starts, n_seqs, out, scale, stretch);
     XRT_LAUNCH_CHECK("attention (prefill)");
     return 0;
-}
-
-template <int HD>
-int launch(const bf16* qkv, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
-           const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
-           const int* seq_starts, int n_seqs, bf16* out, float scale, hipStream_t s) {
-    return launch_waves<HD>(qkv, tokens, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks,
-                            seq_offsets, seq_slots, seq_starts, n_seqs, out, scale, s);
 }
 
 }  // namespace
 
 bool xrt_attention_prefill_accepts(int head_dim) { return head_dim == 64 || head_dim == 128; }
 
-int xrt_attention_prefill(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
+// q_stride: 0, or how far the rows of q lie apart when they hold the queries alone. stretch: 0, or the size of the stretches
+// that positions are cut into (a multiple of the cache block), of which a query sees its own. fine: probabilities of sixteen bits.
+int xrt_attention_prefill(const void* qkv, long q_stride, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                           const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
-                          float scale, hipStream_t s) {
-    if (head_dim == 64)
-        return launch<64>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
-                          block_table, table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, s);
-    return launch<128>((const bf16*)qkv, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache,
-                       block_table, table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, s);
+                          float scale, int stretch, bool fine, hipStream_t s) {
+    XRT_REQUIRE(stretch >= 0 && stretch % BT == 0, "attention (prefill): stretches of %d positions are not whole cache blocks", stretch);
+    XRT_REQUIRE(q_stride == 0 || (q_stride >= (long)n_heads * head_dim && q_stride % 8 == 0 && q_stride <= INT_MAX),
+                "attention (prefill): rows of q %ld apart", q_stride);
+    auto run = [&](auto launcher) {
+        return launcher((const bf16*)qkv, q_stride, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
+                        table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, stretch, s);
+    };
+    if (head_dim == 64) return fine ? run(launch_waves<64, true>) : run(launch_waves<64, false>);
+    return fine ? run(launch_waves<128, true>) : run(launch_waves<128, false>);
 }

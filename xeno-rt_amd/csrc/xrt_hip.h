@@ -286,6 +286,16 @@ int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, i
                           const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
                           int chunk, void* stream);
 
+// The matrix-core attention for a step that brings sequences of many tokens, with the queries alone in q (rows q_stride
+// apart; keys and values are in the cache) and, with chunk > 0, queries that see the keys of their own stretch of `chunk`
+// positions only. `accepts` says which element type, head sizes and stretches it serves (stretches of whole cache blocks).
+// Tokens of the step that belong to no sequence keep what `out` held.
+int xrt_attention_stretches_accepts(int dtype, int head_dim, int value_dim, int chunk);
+int xrt_attention_stretches(const void* q, long q_stride, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                            const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                            const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
+                            float scale, int chunk, void* stream);
+
 // Attention without a softmax: the weight of a visible key is sigmoid(score_h + head_bias[h]), not normalised over the keys;
 // before that the heads' scaled scores of a (query, key) pair are mixed, score_h <- sum_g head_mix[h][g] score_g
 // (head_mix float32 [n_heads][n_heads], or null); a head's summed values are multiplied by sigmoid(gate[token][h]) (float32

@@ -198,7 +198,7 @@ class HipOps:
                      "xrt_attention_general", "xrt_rmsnorm_conv_step", "xrt_attention_sigmoid", "xrt_qkv_complete",
                      "xrt_layernorm", "xrt_layernorm_shift", "xrt_add_layernormed", "xrt_short_conv_with", "xrt_selective_scan",
                      "xrt_bigram_add", "xrt_gated_rows", "xrt_add_weighted", "xrt_glu_clamped", "xrt_softcap", "xrt_cast",
-                     "xrt_route_experts", "xrt_scale_blocks"):
+                     "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -494,6 +494,9 @@ class HipOps:
         from ..cache import BLOCK_TOKENS
         if finish is not None:
             return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
+        if (queries_alone and not sink and distance_bias is None and distance_slopes is None and not window
+                and self._attention_stretches(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, chunk)):
+            return None
         if sink or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone or chunk:
             return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
                                            distance_slopes, sink, distance_bias, queries_alone, chunk)
@@ -529,6 +532,39 @@ class HipOps:
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
             ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
+
+    def _attention_stretches(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, chunk) -> bool:
+        """The matrix-core kernel for a step that brings some sequence several tokens, the queries alone in `q`, every query
+        seeing its own stretch of `chunk` positions (or, chunk None, all keys before it). False: not served here (another
+        element type or head size, stretches that are not whole cache blocks, a step that is not described by sequences, or
+        one token a sequence), and nothing was done."""
+        offsets = getattr(batch, "sequence_offsets", None)
+        seq_slots = getattr(batch, "sequence_slots", None)
+        starts = getattr(batch, "sequence_starts", None)
+        if offsets is None or seq_slots is None or starts is None or int(getattr(batch, "max_count", 0) or 0) <= 1:
+            return False
+        if not self.lib.xrt_attention_stretches_accepts(_code(q), head_dim, value_dim, int(chunk or 0)):
+            return False
+        tokens, n_seqs = q.shape[0], int(batch.n_sequences)
+        if n_seqs <= 0 or n_seqs > tokens:
+            return False
+        q_stride = self._rows(q, "attention q", n_heads * head_dim)
+        self._require(out, "attention out", q.dtype, (tokens, n_heads * head_dim), q)
+        self._require(offsets, "sequence offsets", torch.int32, (n_seqs + 1,), q)
+        self._require(seq_slots, "sequence slots", torch.int32, (n_seqs,), q)
+        self._require(starts, "sequence starts", torch.int32, (n_seqs,), q)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, q, n_kv_heads, head_dim, value_dim)
+        from ..cache import BLOCK_TOKENS
+        if int(batch.max_context) > stride * BLOCK_TOKENS:
+            raise KernelError(f"attention: a sequence of {int(batch.max_context)} tokens exceeds the block table")
+        counts = getattr(batch, "host_counts", None)
+        if counts is None or sum(counts) < tokens:
+            out.zero_()                       # padding rows: written by no one, read by the product that follows
+        self._check(self.lib.xrt_attention_stretches(
+            _ptr(q), ctypes.c_long(q_stride), _code(q), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table),
+            stride, n_blocks, _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs, _ptr(out), ctypes.c_float(scale), int(chunk or 0),
+            self._stream(q)))
+        return True
 
     def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink,
                            distance_bias=None, queries_alone=False, chunk=None):
