@@ -152,6 +152,61 @@ def test_unequal_batches_through_reused_slots(name, dtype, models, engines):
     engine.cache.check()
 
 
+MANY_EXPERTS = {
+    "architecture": "Depunex", "vocab": 80, "width": 64, "norm": {"eps": 1e-5}, "logit_softcap": 12.0,
+    "embedding": {"scale": 2.0, "bigram": {"buckets": 31, "mul_prev": 3, "mul_cur": 5}},
+    "layers": [
+        {"type": "mamba2", "mixer": {"heads": 2, "vdim": 32, "state": 16, "groups": 1, "norm_groups": 2, "conv": 3},
+         "mlp": {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 16, "top": 2, "groups": {"count": 4, "keep": 2}}}},
+        {"type": "parallel",
+         "mixer": {"left": {"heads": 2, "kv_heads": 1, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 128},
+                            "rot": {"dims": 32, "base": 1000.0}},
+                   "right": {"inner": 32, "state": 4, "dt_rank": 2, "conv": 2}, "left_scale": 1.0, "right_scale": 1.0},
+         "mlp": {"kind": "moe", "expert": {"ff": 128}, "router": {"experts": 12, "top": 2}}},
+    ],
+}
+
+
+def test_prompts_long_enough_for_sorted_experts_and_chunks_on_the_matrix_cores(tmp_path):
+    """A model whose experts' widths and whose attention suit the kernels that only steps of many tokens take: prompts of some
+    hundred tokens whole (picks sorted by expert, chunks on the matrix cores), in halves, two in one step and with their ends
+    decoded, against the same engine with every token meeting every expert: the router reads the same rows and chooses the
+    same experts either way, so what differs is rounding alone. (Against the plain model a token whose best scores lie
+    closer than bfloat16 rounds the rows takes another expert, with sixteen experts every thirtieth token or so: there the
+    root mean square is held, and the other tests hold single rows on models with fewer experts.)"""
+    from xeno_rt_amd.engine import Engine
+    folder = make_depunex_folder(MANY_EXPERTS, tmp_path, seed=77)
+    plain = P.PlainModel(folder)
+    requests = [token_ids(MANY_EXPERTS["vocab"], length, seed=length) for length in (300, 281)]
+    engine = Engine.load(folder, dtype="bfloat16", max_tokens=64 * 12, max_slots=2)
+    ops = engine.runtime.ops
+    h = torch.zeros(300, 64, dtype=torch.bfloat16, device="cuda")
+    for layer in engine.model.spec.layers:                       # (the test is about these paths: it says so if they are not taken)
+        mlp = layer.feed_forward
+        assert ops.experts_sorted_takes(h, mlp.w_gate_up, mlp.w_down, mlp.experts, mlp.intermediate, mlp.top)
+    takes = ops.experts_sorted_takes
+    ops.experts_sorted_takes = lambda *operands: False
+    wants = [run_whole(engine, ids) for ids in requests]
+    ops.experts_sorted_takes = takes
+    for ids, want in zip(requests, wants):
+        assert errors(want, plain.logits(ids))[1] <= 5e-2
+
+    def close(got, want, what):
+        # (the second layer's router reads what the first layer's experts made: a rare row may change its experts there too)
+        per_row = (got.double() - want.double()).abs().max(dim=1).values / float(want.abs().max())
+        rms = errors(got, want)[1]
+        assert int((per_row > 4e-2).sum()) <= 3 and rms <= 1e-2, \
+            f"{what}: sorted picks differ from every token with every expert in rows {(per_row > 4e-2).nonzero().flatten().tolist()}, rms {rms:.2e}"
+
+    for ids, want in zip(requests, wants):
+        close(run_whole(engine, ids), want, f"{len(ids)} tokens whole")
+        close(in_portions(engine, ids, [len(ids) // 2 + 1]), want, f"{len(ids)} tokens in halves")
+    for prompts in ([300, 281], [270, 281]):
+        for index, (got, want) in enumerate(zip(run_batched(engine, requests, prompts), wants)):
+            close(got, want, f"batch {prompts} request {index}")
+    engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_greedy_generation_through_the_loop(dtype, models, engines):
     from xeno_rt_amd.engine import GenerateRequest, generate
@@ -568,6 +623,59 @@ def test_an_expert_outside_the_kept_groups_is_never_chosen_however_large_its_sco
     ops.route_experts(logits, weights, 2, 3, 2)
     assert weights[0, 4].item() == 0.0 and weights[0].nonzero().flatten().tolist() == [0, 2]
     assert weights[0, 0].item() == pytest.approx(0.7 / 1.35, rel=1e-5)
+
+
+def expert_operands(ops, tokens, hidden, width, experts, seed, packed_down):
+    generator = torch.Generator().manual_seed(seed)
+    h = torch.randn(tokens, hidden, generator=generator).bfloat16()
+    gates, ups = (0.3 * torch.randn(experts, width, hidden, generator=generator).bfloat16() for _ in range(2))
+    downs = 0.3 * torch.randn(experts, hidden, width, generator=generator).bfloat16()
+    logits = torch.randn(tokens, experts, generator=generator)
+    w_gate_up = ops.pack(torch.cat([gates.reshape(-1, hidden), ups.reshape(-1, hidden)]).cuda(), "gated", gated_n=experts * width)
+    w_down = torch.cat(list(downs), dim=1).contiguous().cuda()
+    return h, gates, ups, downs, logits, w_gate_up, ops.pack(w_down, "tiles") if packed_down else w_down
+
+
+@pytest.mark.parametrize("tokens,hidden,width,experts,top,groups,keep,packed_down", [
+    (300, 64, 64, 8, 2, 4, 2, False), (1000, 128, 192, 16, 4, 1, 1, True), (257, 192, 64, 3, 1, 1, 1, False), (640, 64, 128, 32, 2, 8, 3, True),
+    (129, 320, 64, 5, 5, 1, 1, True)])
+def test_experts_multiply_only_the_tokens_that_chose_them(tokens, hidden, width, experts, top, groups, keep, packed_down, ops):
+    """The picks sorted by expert against the plain sum over every token's experts, against the way in which every token
+    meets every expert, and a token's bits with other tokens around it. (One expert may be chosen by no one, another by all.)"""
+    h, gates, ups, downs, logits, w_gate_up, w_down = expert_operands(ops, tokens, hidden, width, experts, tokens + experts, packed_down)
+    logits[:, 1] -= 30.0                                       # nobody's choice, unless all are chosen
+    weights = torch.empty(tokens, experts, device="cuda")
+    chosen = torch.empty(tokens, top, dtype=torch.int32, device="cuda")
+    ops.route_experts(logits.cuda(), weights, top, groups, keep, chosen=chosen)
+    out = torch.full((tokens, hidden), float("nan"), device="cuda")
+    ops.experts_sorted(h.cuda(), w_gate_up, w_down, weights, chosen, width, out)
+    want = torch.zeros(tokens, hidden, dtype=F)
+    for e in range(experts):
+        takers = (chosen.cpu() == e).any(dim=1)
+        x = h[takers].double()
+        gate, up = x @ gates[e].double().T, x @ ups[e].double().T
+        want[takers] += weights.cpu()[takers, e].double()[:, None] * ((gate * torch.sigmoid(gate) * up) @ downs[e].double().T)
+    assert float((out.double().cpu() - want).abs().max()) <= 1e-2 * float(want.abs().max())
+    # every token with every expert: the same but for the rounding of the weighted activations
+    act = torch.empty(tokens, experts * width, dtype=torch.bfloat16, device="cuda")
+    ops.linear_glu(h.cuda(), w_gate_up, act)
+    ops.scale_blocks(act, weights, width)
+    dense = torch.empty(tokens, hidden, device="cuda")
+    ops.linear(act, w_down, dense)
+    assert float((out - dense).abs().max()) <= 1e-2 * float(want.abs().max())
+    # other company, other rows in the sort: the same bits
+    some = torch.arange(tokens - 1, -1, -3)
+    fewer = torch.empty(len(some), hidden, device="cuda")
+    ops.experts_sorted(h[some].cuda(), w_gate_up, w_down, weights[some.cuda()].contiguous(), chosen[some.cuda()].contiguous(), width, fewer)
+    assert torch.equal(fewer, out[some.cuda()])
+
+
+def test_sorted_experts_are_taken_for_steps_of_many_tokens_only(ops):
+    h, _, _, _, _, w_gate_up, w_down = expert_operands(ops, 512, 64, 64, 8, 1, True)
+    assert ops.experts_sorted_takes(h.cuda(), w_gate_up, w_down, 8, 64, 2)
+    assert not ops.experts_sorted_takes(h[:8].cuda(), w_gate_up, w_down, 8, 64, 2)          # a decode step reads every expert once either way
+    assert not ops.experts_sorted_takes(h.cuda(), w_gate_up, w_down, 8, 64, 8)              # every token uses every expert: nothing to save
+    assert not ops.experts_sorted_takes(h.float().cuda(), w_gate_up, w_down, 8, 64, 2)
 
 
 def test_small_operations(ops):

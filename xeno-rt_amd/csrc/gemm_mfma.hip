@@ -42,7 +42,8 @@ struct RowScale { const float* squares; int tiles; int width; float eps; int act
 template <int BM, int BN, int WM, int WN, int MODE, int DK, int STAGES, typename TO>
 __device__ __forceinline__ void gemm_tile(
     const bf16* __restrict__ a, const bf16* __restrict__ w, TO* __restrict__ out, int M, int N, int K,
-    int id, int tiles_m, int tiles_n, int n_first, int k_per_split, const Packing packing, const RowScale scale = RowScale{}) {
+    int id, int tiles_m, int tiles_n, int n_first, int k_per_split, const Packing packing, const RowScale scale = RowScale{},
+    const int lda = 0, const int ldw = 0) {      // lda, ldw: how far the rows of a and of w lie apart, if not K (whole tiles along k only)
     constexpr int THREADS = WM * WN * XRT_WAVE;
     constexpr int WAVE_M = BM / WM, WAVE_N = BN / WN;        // part of the tile owned by one wavefront
     constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;        // 32x32 accumulator tiles of a wavefront
@@ -143,10 +144,11 @@ __device__ __forceinline__ void gemm_tile(
         const int sub = lane / CHUNKS;                             // row within the rows of one instruction
         auto chunk_of = [&](int row) { return ((lane % CHUNKS) ^ swizzle_of(row)) * 8; };   // what belongs in this lane's place
         unsigned off_a[LOADS_A], off_b[LOADS_B];                   // bytes
+        const long row_a = lda > 0 ? lda : K, row_w = ldw > 0 ? ldw : K;
 #pragma unroll
         for (int i = 0; i < LOADS_A; ++i) {
             const int r = min(i * WAVES + wave, BLOCKS_A - 1) * ROWS + sub;
-            off_a[i] = (unsigned)(min(m0 + r, (long)M - 1) * K + chunk_of(r)) * 2u;
+            off_a[i] = (unsigned)(min(m0 + r, (long)M - 1) * row_a + chunk_of(r)) * 2u;
         }
         // A packed w is copied as it lies: an instruction takes one whole tile of the packing (16 packed rows x 32
         // columns, a contiguous kilobyte, lane by lane), and the stage holds the tile's groups of 16 packed rows
@@ -162,10 +164,10 @@ __device__ __forceinline__ void gemm_tile(
             const int block = min(i * WAVES + wave, BLOCKS_B - 1);
             if (packed_b) {
                 const long group = min(first_packed / 16 + block / 2, last_group);       // groups beyond the matrix: the last one again
-                off_b[i] = (unsigned)(((group * (K / 32) + block % 2) * 512 + lane * 8) * 2);
+                off_b[i] = (unsigned)(((group * (row_w / 32) + block % 2) * 512 + lane * 8) * 2);
             } else {
                 const int r = block * ROWS + sub;
-                off_b[i] = (unsigned)(w_row(r) * K + chunk_of(r)) * 2u;
+                off_b[i] = (unsigned)(w_row(r) * row_w + chunk_of(r)) * 2u;
             }
         }
         // a step of k0 columns along k moves a row contiguous along k by k0 elements, a packed one by k0 / 32 tiles
@@ -479,6 +481,44 @@ __global__ void __launch_bounds__(8 * XRT_WAVE) gemm_mfma_mixed_kernel(
     else
         gemm_tile<128, 256, 2, 4, MODE, 64, 2, TO>(a, w, out, M, N, K, blockIdx.x - large_blocks, small_tiles_m,
                                                    small_tiles_n, split, K, packing, scale);
+}
+
+// Products of groups of rows with matrices of their own (experts): the rows of a stand sorted by group, every group's stretch
+// filled up to whole tiles of GROUPED_BM rows, and tile_group[t] names the group of tile t (negative: the tile holds nothing and
+// its workgroups leave). Group g multiplies with w + g * w_stride; a's rows lie lda apart, w's ldw (so a group's matrix can be
+// some columns of a wider one), K is what is summed over. Grid: x the tiles along n (a whole number of rounds over the XCDs,
+// so that all tiles of one n and one group, which share their w, run on one XCD), z the tiles of rows.
+constexpr int GROUPED_BM = 128, GROUPED_BN = 256;
+template <int MODE, typename TO>
+__global__ void __launch_bounds__(8 * XRT_WAVE) gemm_grouped_kernel(
+    const bf16* __restrict__ a, const bf16* __restrict__ w, long w_stride, TO* __restrict__ out, int N, int K, int lda, int ldw,
+    int tiles_n, const int* __restrict__ tile_group, const Packing packing, const RowScale scale) {
+    const int tile = blockIdx.z;
+    const int group = tile_group[tile];
+    if (group < 0) return;
+    gemm_tile<GROUPED_BM, GROUPED_BN, 2, 4, MODE, 64, 2, TO>(a + (long)tile * GROUPED_BM * lda, w + (long)group * w_stride,
+                                                             out + (long)tile * GROUPED_BM * N, GROUPED_BM, N, K, blockIdx.x, 1, tiles_n, 0, K,
+                                                             packing, scale, lda, ldw);
+}
+
+template <int MODE, typename TO>
+int launch_grouped(const bf16* a, const bf16* w, long w_stride, TO* out, int tiles_m, int N, int K, int lda, int ldw, const int* tile_group,
+                   const Packing& packing, int activation, hipStream_t s) {
+    constexpr int BN_OUT = MODE == MODE_GATED ? GROUPED_BN / 2 : GROUPED_BN;
+    constexpr size_t lds = (size_t)2 * (GROUPED_BM + GROUPED_BN) * 64 * sizeof(bf16);
+    auto kernel = gemm_grouped_kernel<MODE, TO>;
+    static bool configured = false;          // per instantiation
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        XRT_REQUIRE(e == hipSuccess, "linear (groups): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        configured = true;
+    }
+    const int tiles_n = (N + BN_OUT - 1) / BN_OUT;
+    XRT_REQUIRE(tiles_m > 0 && tiles_m <= 65535, "linear (groups): %d tiles of rows", tiles_m);
+    kernel<<<dim3((unsigned)((tiles_n + 7) / 8 * 8), 1, (unsigned)tiles_m), 8 * XRT_WAVE, lds, s>>>(
+        a, w, w_stride, out, N, K, lda, ldw, tiles_n, tile_group, packing, RowScale{nullptr, 0, 0, 0.f, activation});
+    XRT_LAUNCH_CHECK("linear (groups)");
+    return 0;
 }
 
 // Launches the tiles of output columns [n_first, n_first + n_count).
@@ -967,6 +1007,30 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
                     const Packing& packing, hipStream_t s) {
     if (out_dtype == XRT_F32) return launch_shape<float>((const bf16*)a, (const bf16*)w, (float*)out, M, N, K, mode, activation, packing, s);
     return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, activation, packing, s);
+}
+
+// Groups of rows of a, each with a matrix of its own (gemm_grouped_kernel): tiles_m tiles of xrt_linear_groups_tile() rows.
+int xrt_linear_groups_tile() { return GROUPED_BM; }
+
+bool xrt_linear_groups_mfma_accepts(const void* a, int lda, const void* w, int ldw, int N, int K, int mode, const Packing& packing) {
+    const long rows_w = mode == MODE_GATED ? 2L * N : N;
+    if (mode != MODE_STORE && mode != MODE_GATED) return false;
+    if (mode == MODE_GATED && (!is_packed(packing) ? true : packing.kind != XRT_PACK_GATED || packing.gated_n != N || N % 8 != 0)) return false;
+    if (mode == MODE_STORE && is_packed(packing) && packing.kind != XRT_PACK_TILES) return false;
+    return K > 0 && K % 64 == 0 && lda >= K && lda % 8 == 0 && ldw >= K && ldw % (is_packed(packing) ? 32 : 8) == 0 && (uintptr_t)a % 16 == 0 &&
+           (uintptr_t)w % 16 == 0 && (long)GROUPED_BM * lda < (1L << 31) && (rows_w + 15) * ldw < (1L << 31);
+}
+
+int xrt_linear_groups_mfma(const void* a, int lda, const void* w, long w_stride, int ldw, void* out, int out_dtype, int tiles_m, int N, int K,
+                           int mode, int activation, const int* tile_group, const Packing& packing, hipStream_t s) {
+    const bf16* x = (const bf16*)a;
+    const bf16* m = (const bf16*)w;
+    if (mode == MODE_GATED) {
+        if (out_dtype == XRT_F32) return launch_grouped<MODE_GATED, float>(x, m, w_stride, (float*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
+        return launch_grouped<MODE_GATED, bf16>(x, m, w_stride, (bf16*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
+    }
+    if (out_dtype == XRT_F32) return launch_grouped<MODE_STORE, float>(x, m, w_stride, (float*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
+    return launch_grouped<MODE_STORE, bf16>(x, m, w_stride, (bf16*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
 }
 
 // Whether a product runs through the tiles of this section (17 to 64 rows of x, or more rows and few

@@ -198,7 +198,9 @@ class HipOps:
                      "xrt_attention_general", "xrt_rmsnorm_conv_step", "xrt_attention_sigmoid", "xrt_qkv_complete",
                      "xrt_layernorm", "xrt_layernorm_shift", "xrt_add_layernormed", "xrt_short_conv_with", "xrt_selective_scan",
                      "xrt_bigram_add", "xrt_gated_rows", "xrt_add_weighted", "xrt_glu_clamped", "xrt_softcap", "xrt_cast",
-                     "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts"):
+                     "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts",
+                     "xrt_experts_sort", "xrt_gather_rows", "xrt_linear_groups", "xrt_linear_groups_accepts", "xrt_experts_combine",
+                     "xrt_linear_groups_tile_rows"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -212,6 +214,7 @@ class HipOps:
         self.lib.xrt_linear_recurrence_workspace.restype = ctypes.c_long
         self.lib.xrt_attention_sigmoid_workspace.restype = ctypes.c_long
         self.lib.xrt_selective_scan_workspace.restype = ctypes.c_long
+        self.lib.xrt_experts_sort_room.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -976,6 +979,78 @@ class HipOps:
             self._require(chosen, "route_experts chosen", torch.int32, (tokens, top), logits)
         self._check(self.lib.xrt_route_experts(_ptr(logits), ctypes.c_long(tokens), experts, int(top), int(groups), int(keep), int(group_top),
                                                ctypes.c_float(floor), _ptr(weights), _ptr(chosen), self._stream(logits)))
+
+    # -- experts that multiply only the tokens that chose them
+    def _expert_matrices(self, w_gate_up, w_down, experts, width):
+        """(data, packing, elements between two experts' matrices, row distance) of the gate/up matrix and of the down matrix, as
+        `xrt_linear_groups` wants them, or None: [all gates | all ups] packed for a gated epilogue lies expert after expert
+        already (a group of sixteen packed rows holds eight outputs' gate and up rows); an expert's down matrix is `width`
+        columns of the wide one."""
+        if not isinstance(w_gate_up, PackedMatrix) or w_gate_up.packing.kind != PACK_GATED or width % 64 != 0:
+            return None
+        hidden = w_gate_up.shape[1]
+        if w_gate_up.packing.gated_n != experts * width or tuple(w_down.shape) != (hidden, experts * width):
+            return None
+        up = (w_gate_up.data, _Packing(PACK_GATED, width, 0, 0), 2 * width * hidden, hidden)
+        if isinstance(w_down, PackedMatrix):
+            if w_down.packing.kind != PACK_TILES:
+                return None
+            down = (w_down.data, w_down.packing, width * 16, experts * width)
+        else:
+            down = (w_down, None, width, experts * width)
+        return up, down
+
+    def experts_sorted_takes(self, h, w_gate_up, w_down, experts, width, top) -> bool:
+        """Whether `experts_sorted` serves these operands, and pays: it multiplies every pick once, in tiles that are filled up
+        per expert, where the plain way multiplies every token with every expert."""
+        matrices = self._expert_matrices(w_gate_up, w_down, experts, width)
+        if matrices is None or h.dtype != torch.bfloat16 or h.dim() != 2 or h.shape[1] % 64 != 0 or experts > 256:
+            return False
+        tokens, hidden = h.shape
+        room = int(self.lib.xrt_experts_sort_room(ctypes.c_long(tokens), top, experts))
+        if tokens < 64 or 4 * tokens * experts < 5 * room or room // self.group_tile() > 65535:
+            return False
+        (up, up_packing, _, up_rows), (down, down_packing, _, down_rows) = matrices
+        return bool(self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, width, hidden, 2, ctypes.byref(up_packing))
+                    and self.lib.xrt_linear_groups_accepts(_ptr(h), width, _ptr(down), down_rows, hidden, width, 0,
+                                                           None if down_packing is None else ctypes.byref(down_packing)))
+
+    def group_tile(self) -> int:
+        return int(self.lib.xrt_linear_groups_tile_rows())
+
+    def experts_sorted(self, h, w_gate_up, w_down, weights, chosen, width, out, activation: str = "silu"):
+        """out[t] (float32) = sum over the experts e that token t chose, in the order of `chosen`, of weights[t, e] *
+        W_down_e (act(W_gate_e h_t) * (W_up_e h_t)): the picks are sorted by expert, every expert multiplies its own rows, and
+        the outputs go back to their tokens. A token's result does not depend on what else the step holds."""
+        tokens, hidden = h.shape
+        experts, top = weights.shape[1], chosen.shape[1]
+        matrices = self._expert_matrices(w_gate_up, w_down, experts, width)
+        if matrices is None:
+            raise KernelError("experts_sorted: the experts' matrices do not lie expert after expert")
+        (up, up_packing, up_stride, up_rows), (down, down_packing, down_stride, down_rows) = matrices
+        self._require(h, "experts_sorted h", torch.bfloat16)
+        self._require(weights, "experts_sorted weights", torch.float32, (tokens, experts), h)
+        self._require(chosen, "experts_sorted chosen", torch.int32, (tokens, top), h)
+        self._require(out, "experts_sorted out", torch.float32, (tokens, hidden), h)
+        h_stride = self._rows(h, "experts_sorted h", hidden)
+        stream, tile = self._stream(h), self.group_tile()
+        room = int(self.lib.xrt_experts_sort_room(ctypes.c_long(tokens), top, experts))
+        index = self._empty(room + tokens * top + room // tile, torch.int32, h.device)
+        rows, places, tile_group = index[:room], index[room:room + tokens * top], index[room + tokens * top:]
+        self._check(self.lib.xrt_experts_sort(_ptr(chosen), ctypes.c_long(tokens), top, experts, _ptr(rows), ctypes.c_long(room), _ptr(places),
+                                              _ptr(tile_group), stream))
+        gathered = self._empty((room, hidden), torch.bfloat16, h.device)
+        self._check(self.lib.xrt_gather_rows(_ptr(h), ctypes.c_long(h_stride), _ptr(rows), ctypes.c_long(room), hidden, _ptr(gathered), stream))
+        act = self._empty((room, width), torch.bfloat16, h.device)
+        self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows, ctypes.byref(up_packing),
+                                               _ptr(act), _code(act), ctypes.c_long(room // tile), width, hidden,
+                                               2 | (ACTIVATIONS[activation] << 8), _ptr(tile_group), stream))
+        sorted_out = self._empty((room, hidden), torch.float32, h.device)
+        self._check(self.lib.xrt_linear_groups(_ptr(act), width, _ptr(down), ctypes.c_long(down_stride), down_rows,
+                                               None if down_packing is None else ctypes.byref(down_packing), _ptr(sorted_out),
+                                               _code(sorted_out), ctypes.c_long(room // tile), hidden, width, 0, _ptr(tile_group), stream))
+        self._check(self.lib.xrt_experts_combine(_ptr(sorted_out), _ptr(places), _ptr(chosen), _ptr(weights), ctypes.c_long(tokens), top, experts,
+                                                 hidden, _ptr(out), stream))
 
     def scale_blocks(self, act, weights, width):
         """act[t, e * width + c] *= weights[t, e], in place."""

@@ -166,12 +166,14 @@ class Runtime:
             at += tensor.shape[0]
         return out
 
-    def weight(self, tensors, kind: str = "tiles", **details):
+    def weight(self, tensors, kind: str = "tiles", needed: bool = False, **details):
         """What `ops.linear` (or `linear_glu`, `linear_qkv`, `embed`) takes as its w: the matrix (or the matrices
         of equal width, one below the other) in the compute dtype on the device, and, where the kernels have a
         faster layout for matrices of its sizes, in that layout. kind and details name what the product's
         epilogue combines: "tiles" nothing, "gated" gate rows and up rows (gated_n of each), "rotary" the
-        pairs of a rotation over whole heads (head_dim, rotated_heads). Only products read the result."""
+        pairs of a rotation over whole heads (head_dim, rotated_heads). needed: some kernel reads the faster layout as such
+        (not only faster), so it is made wherever it can be, also at sizes where it would not pay by itself. Only products
+        read the result."""
         matrix = self.stacked(tensors) if isinstance(tensors, (list, tuple)) else self.matrix(tensors)
         pack = getattr(self.ops, "pack", None)
         if (pack is None or not self.pack_weights or self.dtype != torch.bfloat16 or matrix.device.type != "cuda"
@@ -181,7 +183,7 @@ class Runtime:
             return matrix
         if kind == "rotary" and details.get("head_dim", 0) % 16 != 0:
             return matrix
-        if self.pack_weights != "always" and not self.ops.packing_suits(matrix.shape[0], matrix.shape[1]):
+        if self.pack_weights != "always" and not needed and not self.ops.packing_suits(matrix.shape[0], matrix.shape[1]):
             return matrix
         return pack(matrix, kind, **details)
 

@@ -147,10 +147,11 @@ class ExpertsMLP(FeedForward):
     best groups can be chosen (groups None: all can); the `top` largest scores are chosen and divided by their sum
     (+ 1e-20) as weights; the output is the weighted sum of the chosen experts' outputs.
 
-    Every expert's gate and up rows lie in one matrix and their down columns in another. A step of many tokens
-    multiplies every token with every expert, weights each expert's stretch of the activations by the router's weight (zero
-    for experts not chosen) and lets the down product add them up: two products of full tiles whatever the choice is, and a
-    token's result never depends on what else the step holds."""
+    Every expert's gate and up rows lie in one matrix and their down columns in another. A step of few tokens multiplies
+    every token with every expert (the step reads all weights once either way), weights each expert's stretch of the
+    activations by the router's weight (zero for experts not chosen) and lets the down product add them up. A step of many
+    tokens sorts its picks by expert, and every expert multiplies the rows that chose it (`ops.experts_sorted`). Either way
+    a token's result never depends on what else the step holds."""
     capturable = True
     GROUP_TOP = 2
     WEIGHT_FLOOR = 1e-20
@@ -178,24 +179,33 @@ class ExpertsMLP(FeedForward):
         super().bind(tensors, runtime)
         self.w_router = runtime.matrix(tensors[self.router_name])
         total = self.experts * self.intermediate
-        # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]
+        # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]; packed for a gated epilogue the
+        # former lies expert after expert, which is what the product of sorted picks reads
         self.w_gate_up = runtime.weight([tensors[names[0]] for names in self.expert_names] + [tensors[names[1]] for names in self.expert_names],
-                                        "gated", gated_n=total)
+                                        "gated", gated_n=total, needed=self.intermediate % 64 == 0 and self.top < self.experts)
         down = torch.empty((self.hidden, total), dtype=runtime.dtype, device=runtime.device)
         for n, names in enumerate(self.expert_names):
             down[:, n * self.intermediate:(n + 1) * self.intermediate].copy_(tensors[names[2]])
         self.w_down = runtime.weight(down)
 
-    def _weights(self, h):
+    def _weights(self, h, chosen=None):
         rt = self.runtime
         logits = rt.empty((h.shape[0], self.experts), torch.float32)
         rt.ops.linear(h, self.w_router, logits)
         weights = rt.empty((h.shape[0], self.experts), torch.float32)
-        rt.ops.route_experts(logits, weights, self.top, self.groups, self.keep, self.GROUP_TOP, self.WEIGHT_FLOOR)
+        rt.ops.route_experts(logits, weights, self.top, self.groups, self.keep, self.GROUP_TOP, self.WEIGHT_FLOOR, chosen=chosen)
         return weights
 
     def forward_into(self, h, batch, out: torch.Tensor) -> None:
         rt = self.runtime
+        # A step of many tokens of which each uses few of the experts: the picks sorted by expert, every expert multiplies the
+        # tokens that chose it. (Where the kernels have no such product, or it would not pay, every token meets every expert.)
+        takes = getattr(rt.ops, "experts_sorted_takes", None)
+        if takes is not None and takes(h, self.w_gate_up, self.w_down, self.experts, self.intermediate, self.top):
+            chosen = rt.empty((h.shape[0], self.top), torch.int32)
+            weights = self._weights(h, chosen)
+            rt.ops.experts_sorted(h, self.w_gate_up, self.w_down, weights, chosen, self.intermediate, out, activation="silu")
+            return
         weights = self._weights(h)
         act = rt.empty((h.shape[0], self.experts * self.intermediate))
         rt.ops.linear_glu(h, self.w_gate_up, act, activation="silu")
