@@ -407,9 +407,7 @@ __global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kerne
         for (int c = threadIdx.x; c < part_width; c += FINISH_THREADS) store_from_float(a.out, dtype, out_at + c0 + c, 0.f);
         return;
     }
-    auto gated = [&](int c) {                              // c: a column of the whole row
-        float sum = raw[out_at + c];
-        for (int part = 1; part < row_split; ++part) sum += raw[(long)part * tokens * width + out_at + c];
+    auto finished = [&](float sum, int c) {                // the parts' sum of column c of the whole row, with the skip and the gate
         if (a.skip != nullptr) sum = fmaf(load_as_float(a.skip, a.skip_dtype, c / a.vdim), load_as_float(a.v, dtype, row * a.v_stride + c), sum);
         if (a.gate != nullptr) {
             const float g = load_as_float(a.gate, a.gate_is_float32 ? XRT_F32 : dtype, row * a.gate_stride + c);
@@ -417,12 +415,30 @@ __global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kerne
         }
         return sum;
     };
+    auto gated = [&](int c) {
+        float sum = raw[out_at + c];
+        for (int part = 1; part < row_split; ++part) sum += raw[(long)part * tokens * width + out_at + c];
+        return finished(sum, c);
+    };
+    // the kept columns' parts are asked for side by side, part after part (a decode step's rows come in many parts, and column
+    // after column every load would wait for the one before it); each column's sum still adds its parts in their order
     float kept[FINISH_KEPT];
     float squares = 0.f;
 #pragma unroll
+    for (int i = 0; i < FINISH_KEPT; ++i) kept[i] = 0.f;
+#pragma unroll 2
+    for (int part = 0; part < row_split; ++part) {
+        const float* from = raw + (long)part * tokens * width + out_at + c0;
+#pragma unroll
+        for (int i = 0; i < FINISH_KEPT; ++i) {
+            const int c = threadIdx.x + i * FINISH_THREADS;
+            if (c < part_width) kept[i] = part == 0 ? from[c] : kept[i] + from[c];
+        }
+    }
+#pragma unroll
     for (int i = 0; i < FINISH_KEPT; ++i) {
         const int c = threadIdx.x + i * FINISH_THREADS;
-        kept[i] = c < part_width ? gated(c0 + c) : 0.f;
+        kept[i] = c < part_width ? finished(kept[i], c0 + c) : 0.f;
         squares = fmaf(kept[i], kept[i], squares);
     }
     for (int c = threadIdx.x + FINISH_KEPT * FINISH_THREADS; c < part_width; c += FINISH_THREADS) { const float o = gated(c0 + c); squares = fmaf(o, o, squares); }
