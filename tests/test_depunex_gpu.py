@@ -638,7 +638,7 @@ def expert_operands(ops, tokens, hidden, width, experts, seed, packed_down):
 
 @pytest.mark.parametrize("tokens,hidden,width,experts,top,groups,keep,packed_down", [
     (300, 64, 64, 8, 2, 4, 2, False), (1000, 128, 192, 16, 4, 1, 1, True), (257, 192, 64, 3, 1, 1, 1, False), (640, 64, 128, 32, 2, 8, 3, True),
-    (129, 320, 64, 5, 5, 1, 1, True)])
+    (129, 320, 64, 5, 5, 1, 1, True), (1700, 64, 128, 4, 2, 2, 1, True)])           # (the last: experts with picks enough for the larger tile)
 def test_experts_multiply_only_the_tokens_that_chose_them(tokens, hidden, width, experts, top, groups, keep, packed_down, ops):
     """The picks sorted by expert against the plain sum over every token's experts, against the way in which every token
     meets every expert, and a token's bits with other tokens around it. (One expert may be chosen by no one, another by all.)"""

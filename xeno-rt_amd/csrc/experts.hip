@@ -15,10 +15,11 @@
 #include "packing.h"
 #include "xrt_hip.h"
 
-int xrt_linear_groups_tile();
+int xrt_linear_groups_tile(long rows, int groups);
 bool xrt_linear_groups_mfma_accepts(const void* a, int lda, const void* w, int ldw, int N, int K, int mode, const Packing& packing);
-int xrt_linear_groups_mfma(const void* a, int lda, const void* w, long w_stride, int ldw, void* out, int out_dtype, int tiles_m, int N, int K,
-                           int mode, int activation, const int* tile_group, const Packing& packing, hipStream_t s);
+int xrt_linear_groups_splits(int tiles_m, int N, int K, int mode);
+int xrt_linear_groups_mfma(const void* a, int lda, const void* w, long w_stride, int ldw, void* out, int out_dtype, int tile, int tiles_m, int N,
+                           int K, int mode, int activation, const int* tile_group, const Packing& packing, int splits, hipStream_t s);
 
 namespace {
 
@@ -162,15 +163,22 @@ __global__ void __launch_bounds__(256) gather_rows_kernel(const bf16* __restrict
 }
 
 // out[t][c] = sum over a token's picks, in their order, of weights[t][expert of the pick] * sorted[row of the pick][c]
+// (sorted: [tiles][parts][tile][width], the parts' sums of a row added in their order first)
 __global__ void __launch_bounds__(256) experts_combine_kernel(const float* __restrict__ sorted, const int* __restrict__ places,
                                                               const int* __restrict__ chosen, const float* __restrict__ weights, int top,
-                                                              int experts, int width, float* __restrict__ out) {
+                                                              int experts, int width, int tile, int parts, float* __restrict__ out) {
     const long t = blockIdx.x;
     for (int c = threadIdx.x * 4; c < width; c += blockDim.x * 4) {
         float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
         for (int k = 0; k < top; ++k) {
             const float w = weights[t * experts + chosen[t * top + k]];
-            const float4 v = *reinterpret_cast<const float4*>(sorted + (long)places[t * top + k] * width + c);
+            const int place = places[t * top + k];
+            const float* row = sorted + (((long)(place / tile) * parts) * tile + place % tile) * width + c;
+            float4 v = *reinterpret_cast<const float4*>(row);
+            for (int part = 1; part < parts; ++part) {
+                const float4 more = *reinterpret_cast<const float4*>(row + (long)part * tile * width);
+                v.x += more.x; v.y += more.y; v.z += more.z; v.w += more.w;
+            }
             sum.x = fmaf(w, v.x, sum.x); sum.y = fmaf(w, v.y, sum.y); sum.z = fmaf(w, v.z, sum.z); sum.w = fmaf(w, v.w, sum.w);
         }
         *reinterpret_cast<float4*>(out + t * width + c) = sum;
@@ -210,11 +218,12 @@ extern "C" int xrt_scale_blocks(void* act, int dtype, const float* weights, long
     return 0;
 }
 
-extern "C" int xrt_linear_groups_tile_rows() { return xrt_linear_groups_tile(); }
+// rows of a tile for a step of `tokens` tokens that choose `top` of `experts` each
+extern "C" int xrt_linear_groups_tile_rows(long tokens, int top, int experts) { return xrt_linear_groups_tile(tokens * top, experts); }
 
 // rows a step's sorted picks need at most: every pick one, and every expert up to a tile less one of filling
 extern "C" long xrt_experts_sort_room(long tokens, int top, int experts) {
-    const long tile = xrt_linear_groups_tile();
+    const long tile = xrt_linear_groups_tile(tokens * top, experts);
     return (tokens * top + (long)experts * (tile - 1) + tile - 1) / tile * tile;
 }
 
@@ -223,7 +232,7 @@ extern "C" int xrt_experts_sort(const int* chosen, long tokens, int top, int exp
     XRT_REQUIRE(chosen && rows && places && tile_group && tokens > 0 && top > 0 && experts > 0 && experts <= XRT_MOST_EXPERTS,
                 "experts_sort: bad operands (%ld tokens, %d of %d experts)", tokens, top, experts);
     XRT_REQUIRE(room == xrt_experts_sort_room(tokens, top, experts) && room < (1L << 30), "experts_sort: room for %ld rows", room);
-    experts_sort_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(chosen, tokens * top, top, experts, xrt_linear_groups_tile(), (int)room, rows, places,
+    experts_sort_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(chosen, tokens * top, top, experts, xrt_linear_groups_tile(tokens * top, experts), (int)room, rows, places,
                                                              tile_group);
     XRT_LAUNCH_CHECK("experts_sort");
     return 0;
@@ -234,19 +243,24 @@ extern "C" int xrt_linear_groups_accepts(const void* a, int lda, const void* w, 
     return xrt_linear_groups_mfma_accepts(a, lda, w, ldw, n, k, mode, packing ? *packing : none) ? 1 : 0;
 }
 
-// out (rows of n, bfloat16 or float32) = for every tile t of xrt_linear_groups_tile_rows() rows of a (bfloat16, rows lda apart)
+// out (rows of n, bfloat16 or float32) = for every tile t of `tile` rows (128 or 256) of a (bfloat16, rows lda apart)
 // with tile_group[t] >= 0: its rows times the matrix at w + tile_group[t] * w_stride (rows ldw apart, k of their columns
 // summed over; packed or not), mode 0, or mode 2 with an activation: act(gate) * up of a packed gated matrix of n pairs.
+// parts: 1, or (mode 0) 2: k is split in two and out holds, tile after tile, the tile's rows of the first half's sums and then
+// those of the second half's, for a reader that adds them (xrt_linear_groups_parts says which pays).
+extern "C" int xrt_linear_groups_parts(long tiles, int n, int k, int coded_mode) { return xrt_linear_groups_splits((int)tiles, n, k, coded_mode & 255); }
+
 extern "C" int xrt_linear_groups(const void* a, int lda, const void* w, long w_stride, int ldw, const xrt_packing* packing, void* out, int out_dtype,
-                                 long tiles, int n, int k, int coded_mode, const int* tile_group, void* stream) {
+                                 int tile, long tiles, int n, int k, int coded_mode, const int* tile_group, int parts, void* stream) {
     const Packing none = {};
     const int mode = coded_mode & 255, activation = coded_mode >> 8;
     XRT_REQUIRE(a && w && out && tile_group && tiles > 0 && tiles <= 65535 && n > 0 && w_stride >= 0, "linear_groups: bad operands");
     XRT_REQUIRE(out_dtype == XRT_F32 || out_dtype == XRT_BF16, "linear_groups: unknown dtype %d", out_dtype);
     XRT_REQUIRE(xrt_linear_groups_mfma_accepts(a, lda, w, ldw, n, k, mode, packing ? *packing : none),
                 "linear_groups: not served (n %d, k %d, rows %d and %d apart, mode %d): k in whole tiles of 64, a gated matrix packed", n, k, lda, ldw, mode);
-    return xrt_linear_groups_mfma(a, lda, w, w_stride, ldw, out, out_dtype, (int)tiles, n, k, mode, activation, tile_group,
-                                  packing ? *packing : none, (hipStream_t)stream);
+    XRT_REQUIRE(parts == 1 || (parts == 2 && mode == 0 && k % 128 == 0), "linear_groups: k in %d parts", parts);
+    return xrt_linear_groups_mfma(a, lda, w, w_stride, ldw, out, out_dtype, tile, (int)tiles, n, k, mode, activation, tile_group,
+                                  packing ? *packing : none, parts, (hipStream_t)stream);
 }
 
 extern "C" int xrt_gather_rows(const void* x, long x_stride, const int* rows, long count, int width, void* out, void* stream) {
@@ -258,10 +272,12 @@ extern "C" int xrt_gather_rows(const void* x, long x_stride, const int* rows, lo
 }
 
 extern "C" int xrt_experts_combine(const float* sorted, const int* places, const int* chosen, const float* weights, long tokens, int top,
-                                   int experts, int width, float* out, void* stream) {
+                                   int experts, int width, int tile, int parts, float* out, void* stream) {
+    XRT_REQUIRE(parts >= 1 && parts <= 2 && tile > 0, "experts_combine: %d parts of tiles of %d rows", parts, tile);
     XRT_REQUIRE(sorted && places && chosen && weights && out && tokens > 0 && tokens < (1L << 31) && top > 0 && experts > 0 && width > 0 &&
                 width % 4 == 0 && (uintptr_t)sorted % 16 == 0 && (uintptr_t)out % 16 == 0, "experts_combine: bad operands");
-    experts_combine_kernel<<<(unsigned)tokens, 256, 0, (hipStream_t)stream>>>(sorted, places, chosen, weights, top, experts, width, out);
+    experts_combine_kernel<<<(unsigned)tokens, 256, 0, (hipStream_t)stream>>>(sorted, places, chosen, weights, top, experts, width,
+                                                                              tile, parts, out);
     XRT_LAUNCH_CHECK("experts_combine");
     return 0;
 }

@@ -484,29 +484,33 @@ __global__ void __launch_bounds__(8 * XRT_WAVE) gemm_mfma_mixed_kernel(
 }
 
 // Products of groups of rows with matrices of their own (experts): the rows of a stand sorted by group, every group's stretch
-// filled up to whole tiles of GROUPED_BM rows, and tile_group[t] names the group of tile t (negative: the tile holds nothing and
+// filled up to whole tiles of BM rows (128, or 256 where the groups are long: the larger tile multiplies half as fast again,
+// and fills up more), and tile_group[t] names the group of tile t (negative: the tile holds nothing and
 // its workgroups leave). Group g multiplies with w + g * w_stride; a's rows lie lda apart, w's ldw (so a group's matrix can be
 // some columns of a wider one), K is what is summed over. Grid: x the tiles along n (a whole number of rounds over the XCDs,
-// so that all tiles of one n and one group, which share their w, run on one XCD), z the tiles of rows.
-constexpr int GROUPED_BM = 128, GROUPED_BN = 256;
-template <int MODE, typename TO>
+// so that all tiles of one n and one group, which share their w, run on one XCD), y the parts that k is split into (each
+// writes its sums to a copy of the tile's outputs: out is [tiles][parts][BM][N] then), z the tiles of rows.
+constexpr int GROUPED_BN = 256;
+template <int BM, int MODE, typename TO>
 __global__ void __launch_bounds__(8 * XRT_WAVE) gemm_grouped_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, long w_stride, TO* __restrict__ out, int N, int K, int lda, int ldw,
     int tiles_n, const int* __restrict__ tile_group, const Packing packing, const RowScale scale) {
     const int tile = blockIdx.z;
     const int group = tile_group[tile];
     if (group < 0) return;
-    gemm_tile<GROUPED_BM, GROUPED_BN, 2, 4, MODE, 64, 2, TO>(a + (long)tile * GROUPED_BM * lda, w + (long)group * w_stride,
-                                                             out + (long)tile * GROUPED_BM * N, GROUPED_BM, N, K, blockIdx.x, 1, tiles_n, 0, K,
-                                                             packing, scale, lda, ldw);
+    // (grid rows split k among them, and gemm_tile puts row y's sums BM * N elements further on: a tile's parts lie one
+    // after the other, tile after tile)
+    gemm_tile<BM, GROUPED_BN, 2, 4, MODE, 64, 2, TO>(a + (long)tile * BM * lda, w + (long)group * w_stride,
+                                                     out + (long)tile * gridDim.y * BM * N, BM, N, K, blockIdx.x, 1, tiles_n,
+                                                     0, K / (int)gridDim.y, packing, scale, lda, ldw);
 }
 
-template <int MODE, typename TO>
+template <int BM, int MODE, typename TO>
 int launch_grouped(const bf16* a, const bf16* w, long w_stride, TO* out, int tiles_m, int N, int K, int lda, int ldw, const int* tile_group,
-                   const Packing& packing, int activation, hipStream_t s) {
+                   const Packing& packing, int activation, int splits, hipStream_t s) {
     constexpr int BN_OUT = MODE == MODE_GATED ? GROUPED_BN / 2 : GROUPED_BN;
-    constexpr size_t lds = (size_t)2 * (GROUPED_BM + GROUPED_BN) * 64 * sizeof(bf16);
-    auto kernel = gemm_grouped_kernel<MODE, TO>;
+    constexpr size_t lds = (size_t)2 * (BM + GROUPED_BN) * 64 * sizeof(bf16);
+    auto kernel = gemm_grouped_kernel<BM, MODE, TO>;
     static bool configured = false;          // per instantiation
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -515,10 +519,22 @@ int launch_grouped(const bf16* a, const bf16* w, long w_stride, TO* out, int til
     }
     const int tiles_n = (N + BN_OUT - 1) / BN_OUT;
     XRT_REQUIRE(tiles_m > 0 && tiles_m <= 65535, "linear (groups): %d tiles of rows", tiles_m);
-    kernel<<<dim3((unsigned)((tiles_n + 7) / 8 * 8), 1, (unsigned)tiles_m), 8 * XRT_WAVE, lds, s>>>(
+    XRT_REQUIRE(splits >= 1 && K % (64 * splits) == 0 && (splits == 1 || MODE == MODE_STORE), "linear (groups): k in %d parts", splits);
+    kernel<<<dim3((unsigned)((tiles_n + 7) / 8 * 8), (unsigned)splits, (unsigned)tiles_m), 8 * XRT_WAVE, lds, s>>>(
         a, w, w_stride, out, N, K, lda, ldw, tiles_n, tile_group, packing, RowScale{nullptr, 0, 0, 0.f, activation});
     XRT_LAUNCH_CHECK("linear (groups)");
     return 0;
+}
+
+template <int BM>
+int launch_grouped_of(const bf16* x, const bf16* m, long w_stride, void* out, int out_dtype, int tiles_m, int N, int K, int lda, int ldw,
+                      const int* tile_group, const Packing& packing, int mode, int activation, int splits, hipStream_t s) {
+    if (mode == MODE_GATED) {
+        if (out_dtype == XRT_F32) return launch_grouped<BM, MODE_GATED, float>(x, m, w_stride, (float*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, splits, s);
+        return launch_grouped<BM, MODE_GATED, bf16>(x, m, w_stride, (bf16*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, splits, s);
+    }
+    if (out_dtype == XRT_F32) return launch_grouped<BM, MODE_STORE, float>(x, m, w_stride, (float*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, splits, s);
+    return launch_grouped<BM, MODE_STORE, bf16>(x, m, w_stride, (bf16*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, splits, s);
 }
 
 // Launches the tiles of output columns [n_first, n_first + n_count).
@@ -1009,8 +1025,9 @@ int xrt_linear_mfma(const void* a, const void* w, void* out, int out_dtype, int 
     return launch_shape<bf16>((const bf16*)a, (const bf16*)w, (bf16*)out, M, N, K, mode, activation, packing, s);
 }
 
-// Groups of rows of a, each with a matrix of its own (gemm_grouped_kernel): tiles_m tiles of xrt_linear_groups_tile() rows.
-int xrt_linear_groups_tile() { return GROUPED_BM; }
+// Groups of rows of a, each with a matrix of its own (gemm_grouped_kernel). The rows of a tile: 256 where a group has some
+// hundred rows on average (the filling of its last tile is then a small part), 128 otherwise.
+int xrt_linear_groups_tile(long rows, int groups) { return groups > 0 && rows / groups >= 384 ? 256 : 128; }
 
 bool xrt_linear_groups_mfma_accepts(const void* a, int lda, const void* w, int ldw, int N, int K, int mode, const Packing& packing) {
     const long rows_w = mode == MODE_GATED ? 2L * N : N;
@@ -1018,19 +1035,24 @@ bool xrt_linear_groups_mfma_accepts(const void* a, int lda, const void* w, int l
     if (mode == MODE_GATED && (!is_packed(packing) ? true : packing.kind != XRT_PACK_GATED || packing.gated_n != N || N % 8 != 0)) return false;
     if (mode == MODE_STORE && is_packed(packing) && packing.kind != XRT_PACK_TILES) return false;
     return K > 0 && K % 64 == 0 && lda >= K && lda % 8 == 0 && ldw >= K && ldw % (is_packed(packing) ? 32 : 8) == 0 && (uintptr_t)a % 16 == 0 &&
-           (uintptr_t)w % 16 == 0 && (long)GROUPED_BM * lda < (1L << 31) && (rows_w + 15) * ldw < (1L << 31);
+           (uintptr_t)w % 16 == 0 && 256L * lda < (1L << 31) && (rows_w + 15) * ldw < (1L << 31);
 }
 
-int xrt_linear_groups_mfma(const void* a, int lda, const void* w, long w_stride, int ldw, void* out, int out_dtype, int tiles_m, int N, int K,
-                           int mode, int activation, const int* tile_group, const Packing& packing, hipStream_t s) {
-    const bf16* x = (const bf16*)a;
-    const bf16* m = (const bf16*)w;
-    if (mode == MODE_GATED) {
-        if (out_dtype == XRT_F32) return launch_grouped<MODE_GATED, float>(x, m, w_stride, (float*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
-        return launch_grouped<MODE_GATED, bf16>(x, m, w_stride, (bf16*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
-    }
-    if (out_dtype == XRT_F32) return launch_grouped<MODE_STORE, float>(x, m, w_stride, (float*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
-    return launch_grouped<MODE_STORE, bf16>(x, m, w_stride, (bf16*)out, tiles_m, N, K, lda, ldw, tile_group, packing, activation, s);
+// How many parts k is best split into: two where the tiles are too few to fill the chip twice over (a last round that is mostly
+// empty costs a whole one), one otherwise. Only plain sums can be split (their parts are added by whoever reads them).
+int xrt_linear_groups_splits(int tiles_m, int N, int K, int mode) {
+    const int tiles_n = (N + GROUPED_BN - 1) / GROUPED_BN;
+    return mode == MODE_STORE && K % 128 == 0 && (long)tiles_m * tiles_n < 2L * XRT_COMPUTE_UNITS ? 2 : 1;
+}
+
+int xrt_linear_groups_mfma(const void* a, int lda, const void* w, long w_stride, int ldw, void* out, int out_dtype, int tile, int tiles_m, int N,
+                           int K, int mode, int activation, const int* tile_group, const Packing& packing, int splits, hipStream_t s) {
+    XRT_REQUIRE(tile == 128 || tile == 256, "linear (groups): tiles of %d rows", tile);
+    if (tile == 256)
+        return launch_grouped_of<256>((const bf16*)a, (const bf16*)w, w_stride, out, out_dtype, tiles_m, N, K, lda, ldw, tile_group, packing, mode,
+                                      activation, splits, s);
+    return launch_grouped_of<128>((const bf16*)a, (const bf16*)w, w_stride, out, out_dtype, tiles_m, N, K, lda, ldw, tile_group, packing, mode,
+                                  activation, splits, s);
 }
 
 // Whether a product runs through the tiles of this section (17 to 64 rows of x, or more rows and few

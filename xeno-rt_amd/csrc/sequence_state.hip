@@ -435,22 +435,54 @@ __global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kerne
             if (c < part_width) kept[i] = part == 0 ? from[c] : kept[i] + from[c];
         }
     }
+    // likewise what the skip and the gate read: every kind of load for all kept columns at once, the element types decided
+    // outside the loops (inside, each column's loads would wait for the column before)
+    auto load_kept = [&](const void* from, bool is_float32, long at, long step, float (&into)[FINISH_KEPT]) {
+        if (is_float32) {
+#pragma unroll
+            for (int i = 0; i < FINISH_KEPT; ++i) {
+                const int c = threadIdx.x + i * FINISH_THREADS;
+                into[i] = c < part_width ? ((const float*)from)[at + (long)c * step] : 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < FINISH_KEPT; ++i) {
+                const int c = threadIdx.x + i * FINISH_THREADS;
+                into[i] = c < part_width ? to_float(((const bf16*)from)[at + (long)c * step]) : 0.f;
+            }
+        }
+    };
+    if (a.skip != nullptr) {
+        float values[FINISH_KEPT];
+        load_kept(a.v, dtype == XRT_F32, row * a.v_stride + c0, 1, values);
+#pragma unroll
+        for (int i = 0; i < FINISH_KEPT; ++i) {
+            const int c = min(threadIdx.x + i * FINISH_THREADS, part_width - 1);
+            kept[i] = fmaf(load_as_float(a.skip, a.skip_dtype, (c0 + c) / a.vdim), values[i], kept[i]);
+        }
+    }
+    if (a.gate != nullptr) {
+        float gates[FINISH_KEPT];
+        load_kept(a.gate, a.gate_is_float32 || dtype == XRT_F32, row * a.gate_stride + c0, 1, gates);
+#pragma unroll
+        for (int i = 0; i < FINISH_KEPT; ++i) kept[i] *= a.gate_act == XRT_GATE_SILU ? silu_exact(gates[i]) : gates[i];
+    }
 #pragma unroll
     for (int i = 0; i < FINISH_KEPT; ++i) {
         const int c = threadIdx.x + i * FINISH_THREADS;
-        kept[i] = c < part_width ? finished(kept[i], c0 + c) : 0.f;
+        if (c >= part_width) kept[i] = 0.f;
         squares = fmaf(kept[i], kept[i], squares);
     }
     for (int c = threadIdx.x + FINISH_KEPT * FINISH_THREADS; c < part_width; c += FINISH_THREADS) { const float o = gated(c0 + c); squares = fmaf(o, o, squares); }
     const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)part_width + a.eps);
+    float weights[FINISH_KEPT];
+#pragma unroll
+    for (int i = 0; i < FINISH_KEPT; ++i) weights[i] = 1.f;
+    if (a.norm_weight != nullptr) load_kept(a.norm_weight, a.norm_weight_dtype == XRT_F32, c0, 1, weights);
 #pragma unroll
     for (int i = 0; i < FINISH_KEPT; ++i) {
         const int c = threadIdx.x + i * FINISH_THREADS;
-        if (c < part_width) {
-            float value = kept[i] * inv;
-            if (a.norm_weight != nullptr) value *= load_as_float(a.norm_weight, a.norm_weight_dtype, c0 + c);
-            store_from_float(a.out, dtype, out_at + c0 + c, value);
-        }
+        if (c < part_width) store_from_float(a.out, dtype, out_at + c0 + c, kept[i] * inv * weights[i]);
     }
     for (int c = threadIdx.x + FINISH_KEPT * FINISH_THREADS; c < part_width; c += FINISH_THREADS) {
         float value = gated(c0 + c) * inv;

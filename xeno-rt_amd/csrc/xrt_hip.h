@@ -398,22 +398,25 @@ int xrt_route_experts(const float* logits, long tokens, int experts, int top, in
 int xrt_scale_blocks(void* act, int dtype, const float* weights, long tokens, int experts, int width, void* stream);
 
 // Experts that multiply only the tokens that chose them. xrt_experts_sort puts a step's picks (chosen [tokens][top]) in the
-// order of their experts, every expert's stretch filled up to whole tiles of xrt_linear_groups_tile_rows() rows: rows [room]
+// order of their experts, every expert's stretch filled up to whole tiles of xrt_linear_groups_tile_rows() rows (128, or 256 where an expert has some hundred picks on average): rows [room]
 // takes the token of every row (-1: filling), places [tokens][top] the row of every pick, tile_group [room / tile] the expert
 // of every tile (-1: beyond the last); room is xrt_experts_sort_room(). xrt_gather_rows copies rows of bfloat16 x (zeros
 // where rows[r] < 0). xrt_linear_groups multiplies every tile of rows of a with the matrix of its tile's group, w + group *
 // w_stride (elements), whose rows lie ldw apart and of which k columns are summed over (coded_mode as in xrt_linear_with: 0,
 // or 2 | activation << 8 with a packed gated matrix of n pairs per group); `accepts` says what it serves.
 // xrt_experts_combine: out[t] = sum over the picks of t, in their order, of weights[t][chosen[t][k]] * sorted[places[t][k]].
-int xrt_linear_groups_tile_rows();
+int xrt_linear_groups_tile_rows(long tokens, int top, int experts);
 long xrt_experts_sort_room(long tokens, int top, int experts);
 int xrt_experts_sort(const int* chosen, long tokens, int top, int experts, int* rows, long room, int* places, int* tile_group, void* stream);
 int xrt_gather_rows(const void* x, long x_stride, const int* rows, long count, int width, void* out, void* stream);
 int xrt_linear_groups_accepts(const void* a, int lda, const void* w, int ldw, int n, int k, int mode, const xrt_packing* packing);
+// parts: 1, or with plain sums 2: k in two halves whose sums lie tile after tile, [tiles][parts][tile rows][n], for
+// xrt_experts_combine to add (xrt_linear_groups_parts: which of the two pays, from the number of tiles).
+int xrt_linear_groups_parts(long tiles, int n, int k, int coded_mode);
 int xrt_linear_groups(const void* a, int lda, const void* w, long w_stride, int ldw, const xrt_packing* packing, void* out, int out_dtype,
-                      long tiles, int n, int k, int coded_mode, const int* tile_group, void* stream);
+                      int tile, long tiles, int n, int k, int coded_mode, const int* tile_group, int parts, void* stream);
 int xrt_experts_combine(const float* sorted, const int* places, const int* chosen, const float* weights, long tokens, int top, int experts,
-                        int width, float* out, void* stream);
+                        int width, int tile, int parts, float* out, void* stream);
 
 #ifdef __cplusplus
 }

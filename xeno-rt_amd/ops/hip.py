@@ -200,7 +200,7 @@ class HipOps:
                      "xrt_bigram_add", "xrt_gated_rows", "xrt_add_weighted", "xrt_glu_clamped", "xrt_softcap", "xrt_cast",
                      "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts",
                      "xrt_experts_sort", "xrt_gather_rows", "xrt_linear_groups", "xrt_linear_groups_accepts", "xrt_experts_combine",
-                     "xrt_linear_groups_tile_rows"):
+                     "xrt_linear_groups_tile_rows", "xrt_linear_groups_parts"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -1008,15 +1008,16 @@ class HipOps:
             return False
         tokens, hidden = h.shape
         room = int(self.lib.xrt_experts_sort_room(ctypes.c_long(tokens), top, experts))
-        if tokens < 64 or 4 * tokens * experts < 5 * room or room // self.group_tile() > 65535:
+        if tokens < 64 or 4 * tokens * experts < 5 * room or room // 128 > 65535:
             return False
         (up, up_packing, _, up_rows), (down, down_packing, _, down_rows) = matrices
         return bool(self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, width, hidden, 2, ctypes.byref(up_packing))
                     and self.lib.xrt_linear_groups_accepts(_ptr(h), width, _ptr(down), down_rows, hidden, width, 0,
                                                            None if down_packing is None else ctypes.byref(down_packing)))
 
-    def group_tile(self) -> int:
-        return int(self.lib.xrt_linear_groups_tile_rows())
+    def group_tile(self, tokens: int, top: int, experts: int) -> int:
+        """Rows of a tile of sorted picks for a step of that many tokens."""
+        return int(self.lib.xrt_linear_groups_tile_rows(ctypes.c_long(tokens), int(top), int(experts)))
 
     def experts_sorted(self, h, w_gate_up, w_down, weights, chosen, width, out, activation: str = "silu"):
         """out[t] (float32) = sum over the experts e that token t chose, in the order of `chosen`, of weights[t, e] *
@@ -1033,7 +1034,7 @@ class HipOps:
         self._require(chosen, "experts_sorted chosen", torch.int32, (tokens, top), h)
         self._require(out, "experts_sorted out", torch.float32, (tokens, hidden), h)
         h_stride = self._rows(h, "experts_sorted h", hidden)
-        stream, tile = self._stream(h), self.group_tile()
+        stream, tile = self._stream(h), self.group_tile(tokens, top, experts)
         room = int(self.lib.xrt_experts_sort_room(ctypes.c_long(tokens), top, experts))
         index = self._empty(room + tokens * top + room // tile, torch.int32, h.device)
         rows, places, tile_group = index[:room], index[room:room + tokens * top], index[room + tokens * top:]
@@ -1043,14 +1044,16 @@ class HipOps:
         self._check(self.lib.xrt_gather_rows(_ptr(h), ctypes.c_long(h_stride), _ptr(rows), ctypes.c_long(room), hidden, _ptr(gathered), stream))
         act = self._empty((room, width), torch.bfloat16, h.device)
         self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows, ctypes.byref(up_packing),
-                                               _ptr(act), _code(act), ctypes.c_long(room // tile), width, hidden,
-                                               2 | (ACTIVATIONS[activation] << 8), _ptr(tile_group), stream))
-        sorted_out = self._empty((room, hidden), torch.float32, h.device)
+                                               _ptr(act), _code(act), tile, ctypes.c_long(room // tile), width, hidden,
+                                               2 | (ACTIVATIONS[activation] << 8), _ptr(tile_group), 1, stream))
+        # (few tiles: the sum over an expert's width in two halves, which the last kernel adds)
+        parts = int(self.lib.xrt_linear_groups_parts(ctypes.c_long(room // tile), hidden, width, 0))
+        sorted_out = self._empty((room * parts, hidden), torch.float32, h.device)
         self._check(self.lib.xrt_linear_groups(_ptr(act), width, _ptr(down), ctypes.c_long(down_stride), down_rows,
                                                None if down_packing is None else ctypes.byref(down_packing), _ptr(sorted_out),
-                                               _code(sorted_out), ctypes.c_long(room // tile), hidden, width, 0, _ptr(tile_group), stream))
+                                               _code(sorted_out), tile, ctypes.c_long(room // tile), hidden, width, 0, _ptr(tile_group), parts, stream))
         self._check(self.lib.xrt_experts_combine(_ptr(sorted_out), _ptr(places), _ptr(chosen), _ptr(weights), ctypes.c_long(tokens), top, experts,
-                                                 hidden, _ptr(out), stream))
+                                                 hidden, tile, parts, _ptr(out), stream))
 
     def scale_blocks(self, act, weights, width):
         """act[t, e * width + c] *= weights[t, e], in place."""
