@@ -161,7 +161,7 @@ def depunex_config(size, layers, max_positions):
     kinds = [{"type": "mamba2", "mixer": duality, "mlp": dense}, {"type": "parallel", "mixer": pair, "mlp": experts},
              {"type": "mamba2", "mixer": duality, "mlp": experts}, {"type": "parallel", "mixer": pair, "mlp": dense}]
     return {"architecture": "Depunex", "vocab": size["vocab"], "width": w, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
-            "embedding": {"scale": w ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "token_side": {"dim": 64},
+            "embedding": {"scale": w ** 0.5, "bigram": {"buckets": 65521, "mul_prev": 131, "mul_cur": 29}}, "token_side": {"dim": 64},
             "layers": [kinds[i % 4] for i in range(layers)]}
 
 
