@@ -65,7 +65,7 @@ EDGES = {
 CONFIGS = {"mixed": MIXED, "wide": WIDE, "edges": EDGES}
 
 
-def make_depunex_folder(raw_config, folder, seed, std=0.2):
+def make_depunex_folder(raw_config, folder, seed, std=0.2, router_std=0.5):
     """A model folder for `raw_config` with the library's random weights, where the small tensors are then given values that
     make them matter: gains and layer scales away from one, biases and skips away from zero, step sizes and decay rates in
     the range where a state neither forgets at once nor keeps everything, a router whose scores differ."""
@@ -95,7 +95,7 @@ def make_depunex_folder(raw_config, folder, seed, std=0.2):
         elif last == "A_log":
             new = normal(tensor.shape, -1.0, 1.0)
         elif last == "router":
-            new = normal(tensor.shape, 0.0, 0.5)
+            new = normal(tensor.shape, 0.0, router_std)      # (wide models take a smaller one: a sigmoid of 17 is 1.0 in float32)
         elif name in ("bigram", "side.embed"):
             new = normal(tensor.shape, 0.0, 0.5)
         else:

@@ -820,6 +820,72 @@ def test_configurations_drawn_at_random(seed, tmp_path):
         engine.cache.check()
 
 
+def random_configuration_for_long_steps(seed):
+    """Sizes that the kernels for steps of many tokens serve (heads of 64 or 128 whose values are as wide, chunks of whole cache
+    blocks, experts' widths and a model width in multiples of 64, many experts of which few are chosen), mixed with some that
+    they do not serve."""
+    import random
+    r = random.Random(1000 + seed)
+    width = r.choice([64, 128, 192])
+    layers = []
+    for index in range(r.randint(2, 3)):
+        if index % 2 == seed % 2:
+            heads = r.randint(1, 3)
+            mixer = {"heads": heads, "vdim": r.choice([16, 32]), "state": r.choice([8, 32]), "groups": 1, "norm_groups": r.choice([1, heads]),
+                     "conv": r.randint(2, 4)}
+            kind = "mamba2"
+        else:
+            kv_heads, dim = r.randint(1, 2), r.choice([64, 128])
+            left = {"heads": kv_heads * r.randint(1, 2), "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
+            if r.random() < 0.8:
+                left["mask"] = {"size": r.choice([64, 128, 192, 100])}
+            left["rot"] = {"dims": r.choice([16, dim // 2, dim]), "base": 10000.0}
+            mixer = {"left": left, "right": {"inner": 32, "state": 4, "dt_rank": 2, "conv": 3}, "left_scale": 1.0, "right_scale": 0.5}
+            kind = "parallel"
+        count = r.choice([1, 2, 4])
+        per = r.choice([3, 4, 6])
+        router = {"experts": count * per, "top": r.randint(1, 2)}
+        if count > 1:
+            router["groups"] = {"count": count, "keep": r.randint(1, count)}
+        layers.append({"type": kind, "mixer": mixer, "mlp": {"kind": "moe", "expert": {"ff": r.choice([64, 128, 48])}, "router": router}})
+    return {"architecture": "Depunex", "vocab": 90, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 2.0}, "logit_softcap": 20.0,
+            "layers": layers}
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_configurations_drawn_at_random_for_steps_of_many_tokens(seed, tmp_path):
+    """In float32 against the plain model; in bfloat16 the kernels that only steps of many tokens take (sorted experts, chunks
+    on the matrix cores) against the same engine without them, which chooses the same experts from the same rows."""
+    from xeno_rt_amd.engine import Engine
+    raw = random_configuration_for_long_steps(seed)
+    folder = make_depunex_folder(raw, tmp_path / "model", seed=seed, std=0.1, router_std=0.08)
+    plain = P.PlainModel(folder)
+    requests = [token_ids(raw["vocab"], length, seed=seed + length) for length in (330, 290)]
+    engine = Engine.load(folder, dtype="float32", max_tokens=64 * 12, max_slots=2)
+    for ids in requests:
+        assert_logits(run_whole(engine, ids), plain.logits(ids), "float32", f"drawn for long steps {seed}, {len(ids)} tokens")
+    del engine
+    engine = Engine.load(folder, dtype="bfloat16", max_tokens=64 * 12, max_slots=2)
+    ops = engine.runtime.ops
+    fast = (ops.experts_sorted_takes, ops._attention_stretches)
+    ops.experts_sorted_takes, ops._attention_stretches = (lambda *operands: False), (lambda *operands: False)
+    wants = [run_whole(engine, ids) for ids in requests]
+    ops.experts_sorted_takes, ops._attention_stretches = fast
+
+    def close(got, want, what):
+        per_row = (got.double() - want.double()).abs().max(dim=1).values / float(want.abs().max())
+        rms = errors(got, want)[1]
+        assert int((per_row > 5e-2).sum()) <= max(3, len(per_row) // 50) and rms <= 1.5e-2, \
+            f"drawn for long steps {seed}, {what}: rows {(per_row > 5e-2).nonzero().flatten().tolist()} differ, rms {rms:.2e}"
+
+    for ids, want in zip(requests, wants):
+        close(run_whole(engine, ids), want, f"{len(ids)} tokens whole")
+        close(in_portions(engine, ids, [200, 100, 1]), want, f"{len(ids)} tokens in portions")
+    for index, (got, want) in enumerate(zip(run_batched(engine, requests, [330, 280]), wants)):
+        close(got, want, f"batched, request {index}")
+    engine.cache.check()
+
+
 def test_zz_the_largest_errors_seen_are_reported():
     for dtype, (worst, rms) in WORST.items():
         print(f"depunex {dtype}: largest max error {worst:.3e}, largest rms error {rms:.3e}")

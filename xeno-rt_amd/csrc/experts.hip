@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(64) route_experts_kernel(const float* __restri
         for (int round = 0; round < keep; ++round) {
             int best = -1;
             for (int g = 0; g < groups; ++g)
-                if (group_score[g] >= 0.f && (best < 0 || group_score[g] > group_score[best])) best = g;
+                if (!(group_score[g] < 0.f) && (best < 0 || group_score[g] > group_score[best])) best = g;    // (a score that is no number still stands for its group)
             group_score[best] = -1.f;                              // (scores are sums of sigmoids: never negative)
             for (int i = 0; i < per_group; ++i) open[best * per_group + i] = 1;
         }
