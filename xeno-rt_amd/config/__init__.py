@@ -280,7 +280,7 @@ def registered_architectures():
 
 def _ensure_builtin() -> None:
     # The built-in architectures register themselves when their module is imported.
-    from ..models import depunex, ledudra, llama, sozopel  # noqa: F401
+    from ..models import depunex, ledudra, llama, renapel, sozopel  # noqa: F401
 
 
 def parse_config(raw: dict):

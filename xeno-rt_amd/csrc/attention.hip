@@ -8,8 +8,8 @@
 int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
-                          int window, const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
-                          int chunk, hipStream_t s);
+                          int window, const float* distance_slopes, int sink, const float* sink_scores, long q_stride,
+                          const float* distance_bias, int bias_span, int chunk, hipStream_t s);
 bool xrt_attention_decode_accepts(int head_dim);
 long xrt_attention_decode_workspace(int tokens, int n_heads, int n_kv_heads, int head_dim, int max_context);
 int xrt_attention_decode(const void* qkv, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
@@ -66,7 +66,7 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
         }
     }
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, head_dim, k_cache, v_cache, block_table,
-                                 table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, 0, 0, nullptr, 0, 0, s);
+                                 table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, 0, nullptr, 0, nullptr, 0, 0, s);
 }
 
 // The general kernel asked for by name, with what only it serves: values of another width than the keys (qkv rows are
@@ -80,17 +80,18 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
 extern "C" int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                                      const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                                      const int* positions, const int* slots, void* out, float scale, int window,
-                                     const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
-                                     int chunk, void* stream) {
+                                     const float* distance_slopes, int sink, const float* sink_scores, long q_stride,
+                                     const float* distance_bias, int bias_span, int chunk, void* stream) {
     XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention: head counts %d/%d: the first must be a multiple of the second", n_heads, n_kv_heads);
     XRT_REQUIRE(head_dim > 0 && value_dim > 0, "attention: head sizes %d and %d must be positive", head_dim, value_dim);
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "attention: unknown dtype %d", dtype);
     XRT_REQUIRE(qkv && k_cache && v_cache && block_table && positions && slots && out, "attention: null operand");
     XRT_REQUIRE(table_stride > 0 && n_blocks > 0 && window >= 0 && chunk >= 0, "attention: empty cache, or negative window or chunk");
+    XRT_REQUIRE(sink || sink_scores == nullptr, "attention: the sink's scores without a sink");
     if (tokens == 0) return 0;
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, value_dim, k_cache, v_cache, block_table,
-                                 table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, sink, q_stride,
+                                 table_stride, n_blocks, positions, slots, out, scale, window, distance_slopes, sink, sink_scores, q_stride,
                                  distance_bias, bias_span, chunk, (hipStream_t)stream);
 }
 

@@ -194,8 +194,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim, int value_dim,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
-    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink, int chunk_blocks,
-    const float* __restrict__ distance_bias, int bias_span, int stretch) {
+    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink,
+    const float* __restrict__ sink_scores, int chunk_blocks, const float* __restrict__ distance_bias, int bias_span, int stretch) {
     __shared__ float qs[G * OWNED * XRT_WAVE];                 // [G][head_dim]
     __shared__ float ps[WAVES][G * XRT_WAVE];
     // what the wavefronts found in the chunks of a round, for the merge: two sets, used in turn (WAVES > 1)
@@ -281,10 +281,10 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        if (sink) {                                            // one more key, whose score is 0 and whose value is nothing
+        if (sink) {                                            // one more key, whose value is nothing; its score is 0, or the head's own number
             Seen<OWNED> nothing;
             nothing.clear();
-            nothing.m = 0.f;
+            nothing.m = sink_scores != nullptr ? sink_scores[head0 + g] : 0.f;
             nothing.l = 1.f;
             merge(all[g], nothing);
         }
@@ -302,8 +302,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
 int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
-                          int window, const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
-                          int stretch, hipStream_t s) {
+                          int window, const float* distance_slopes, int sink, const float* sink_scores, long q_stride,
+                          const float* distance_bias, int bias_span, int stretch, hipStream_t s) {
     XRT_REQUIRE(distance_bias == nullptr || bias_span > 0, "attention: a table of biases by distance needs a distance at least");
     XRT_REQUIRE(head_dim <= MAX_HEAD_DIM && value_dim > 0 && value_dim <= MAX_HEAD_DIM, "attention: head sizes %d and %d must be at most %d", head_dim, value_dim, MAX_HEAD_DIM);
     // Query heads of a key/value head that a wavefront takes together: as many of the group as 4, for head sizes up to 128
@@ -325,7 +325,7 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
 #define XRT_GENERIC(T, WAVES_, G_, OWNED_)                                                                                \
     attention_generic_kernel<T, WAVES_, G_, OWNED_><<<(unsigned)items, WAVES_ * XRT_WAVE, WAVES_ > 1 ? round_bytes : 0, s>>>( \
         (const T*)qkv, row_width, n_heads, n_kv_heads, head_dim, value_dim, (const T*)k_cache, (const T*)v_cache, block_table,       \
-        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, chunk_blocks, distance_bias, bias_span, stretch)
+        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, sink_scores, chunk_blocks, distance_bias, bias_span, stretch)
 #define XRT_GENERIC_WAVES(T, G_, OWNED_) do { if (side_by_side) XRT_GENERIC(T, CHUNK_WAVES, G_, OWNED_); else XRT_GENERIC(T, 1, G_, OWNED_); } while (0)
 #define XRT_GENERIC_SETS(T)                                                                                               \
     do {                                                                                                                  \

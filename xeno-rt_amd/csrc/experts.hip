@@ -1,5 +1,6 @@
 // Choosing experts for every token, and weighting what the experts made.
-//   xrt_route_experts   from router logits z [tokens][experts] (float32): scores s = sigmoid(z); the experts stand in `groups`
+//   xrt_route_experts   from router logits z [tokens][experts] (float32): scores s = sigmoid(z), or softmax(z) over all experts
+//                       (softmax != 0); the chosen weights are multiplied by `scale` in the end; the experts stand in `groups`
 //                       equal groups of neighbours, a group's score is the sum of its `group_top` largest scores, only experts
 //                       of the `keep` best groups can be chosen; the `top` largest scores among those are chosen, and their
 //                       weights are their scores divided by the scores' sum (+ floor). Equal scores: the lower index wins.
@@ -31,14 +32,20 @@ __device__ __forceinline__ void store_from_float(void* p, int dtype, long i, flo
 }
 
 __global__ void __launch_bounds__(64) route_experts_kernel(const float* __restrict__ logits, long tokens, int experts, int top, int groups, int keep,
-                                                           int group_top, float floor_, float* __restrict__ weights, int* __restrict__ chosen) {
+                                                           int group_top, float floor_, float* __restrict__ weights, int* __restrict__ chosen,
+                                                           int softmax, float scale) {
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= tokens) return;
     float s[XRT_MOST_EXPERTS];
     unsigned char open[XRT_MOST_EXPERTS];          // 1: may still be chosen
     const int per_group = experts / groups;
+    float top_logit = -INFINITY, total = 0.f;
+    if (softmax) {
+        for (int e = 0; e < experts; ++e) top_logit = fmaxf(top_logit, logits[t * experts + e]);
+        for (int e = 0; e < experts; ++e) total += expf(logits[t * experts + e] - top_logit);
+    }
     for (int e = 0; e < experts; ++e) {
-        s[e] = 1.0f / (1.0f + expf(-logits[t * experts + e]));
+        s[e] = softmax ? expf(logits[t * experts + e] - top_logit) / total : 1.0f / (1.0f + expf(-logits[t * experts + e]));
         open[e] = groups > 1 ? 0 : 1;
     }
     if (groups > 1) {
@@ -78,7 +85,7 @@ __global__ void __launch_bounds__(64) route_experts_kernel(const float* __restri
         sum += s[best];
     }
     for (int round = 0; round < top; ++round) {
-        weights[t * experts + picks[round]] = s[picks[round]] / (sum + floor_);
+        weights[t * experts + picks[round]] = s[picks[round]] / (sum + floor_) * scale;
         if (chosen != nullptr) chosen[t * top + round] = picks[round];
     }
 }
@@ -188,7 +195,7 @@ __global__ void __launch_bounds__(256) experts_combine_kernel(const float* __res
 }  // namespace
 
 extern "C" int xrt_route_experts(const float* logits, long tokens, int experts, int top, int groups, int keep, int group_top, float floor_,
-                                 float* weights, int* chosen, void* stream) {
+                                 float* weights, int* chosen, int softmax, float scale, void* stream) {
     XRT_REQUIRE(logits && weights && tokens >= 0, "route_experts: null operand");
     XRT_REQUIRE(experts > 0 && experts <= XRT_MOST_EXPERTS && top > 0 && groups > 0 && experts % groups == 0 && keep > 0 && keep <= groups &&
                 group_top > 0 && (groups == 1 || experts / groups <= 128) && top <= keep * (experts / groups),
@@ -196,7 +203,7 @@ extern "C" int xrt_route_experts(const float* logits, long tokens, int experts, 
                 "chosen than the kept groups hold", experts, groups, keep, top, XRT_MOST_EXPERTS);
     if (tokens == 0) return 0;
     route_experts_kernel<<<(unsigned)((tokens + 63) / 64), 64, 0, (hipStream_t)stream>>>(logits, tokens, experts, top, groups, keep, group_top,
-                                                                                       floor_, weights, chosen);
+                                                                                       floor_, weights, chosen, softmax, scale);
     XRT_LAUNCH_CHECK("route_experts");
     return 0;
 }

@@ -196,12 +196,16 @@ __device__ __forceinline__ void load_token(TokenInputs<M>& in, const xrt_recurre
         in.q[m] = 0.f; in.k[m] = 0.f; in.d[m] = 1.f;
         if (i < rows) {
             const long at = (long)head * a.dim + row0 + i, qk_at = (long)qk_head * a.dim + row0 + i;
-            in.q[m] = load_as_float(a.q, dtype, row * a.q_stride + qk_at) * a.q_scale;
-            in.k[m] = load_as_float(a.k, dtype, row * a.k_stride + qk_at) * a.k_scale;
+            float q = load_as_float(a.q, dtype, row * a.q_stride + qk_at), k = load_as_float(a.k, dtype, row * a.k_stride + qk_at);
+            if (a.input_silu) { q = silu_exact(q); k = silu_exact(k); }
+            in.q[m] = q * a.q_scale;
+            in.k[m] = k * a.k_scale;
             in.d[m] = stepped ? stepped_decay : decay_of(a, row, head, at);
         }
     }
-    in.v = owner ? load_as_float(a.v, dtype, row * a.v_stride + (long)head * a.vdim + column) * step : 0.f;
+    float v = owner ? load_as_float(a.v, dtype, row * a.v_stride + (long)head * a.vdim + column) : 0.f;
+    if (a.input_silu) v = silu_exact(v);
+    in.v = v * step;
 }
 
 // grid (sequences, heads * vslices * row_split, segments), one wavefront each. With row_split > 1 (one segment only) a wavefront
@@ -346,6 +350,10 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_combine_kernel(const xrt_
     }
 }
 
+__device__ __forceinline__ float gate_value(float g, int act) {
+    return act == XRT_GATE_SILU ? silu_exact(g) : act == XRT_GATE_SIGMOID ? 1.0f / (1.0f + expf(-g)) : g;
+}
+
 // The heads' raw outputs of one token: norm over vdim, weight, gate. A wavefront per (token, head).
 __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_recurrence a, int dtype, const float* __restrict__ raw,
                                                                     const int* __restrict__ token_slots, int row_split, long tokens) {
@@ -386,7 +394,7 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_r
             value *= load_as_float(a.norm_weight, a.norm_weight_dtype, a.norm_weight_per_head ? (long)head * vdim + c : c);
         if (a.gate != nullptr) {
             const float g = load_as_float(a.gate, a.gate_is_float32 ? XRT_F32 : dtype, row * a.gate_stride + (long)head * vdim + c);
-            value *= a.gate_act == XRT_GATE_SILU ? silu_exact(g) : g;
+            value *= gate_value(g, a.gate_act);
         }
         store_from_float(a.out, dtype, out_at + c, value);
     }
@@ -409,11 +417,15 @@ __global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kerne
     }
     auto finished = [&](float sum, int c) {                // the parts' sum of column c of the whole row, with the skip and the gate
         if (a.skip != nullptr) sum = fmaf(load_as_float(a.skip, a.skip_dtype, c / a.vdim), load_as_float(a.v, dtype, row * a.v_stride + c), sum);
-        if (a.gate != nullptr) {
+        if (a.gate != nullptr && !a.gate_after_norm) {
             const float g = load_as_float(a.gate, a.gate_is_float32 ? XRT_F32 : dtype, row * a.gate_stride + c);
-            sum *= a.gate_act == XRT_GATE_SILU ? silu_exact(g) : g;
+            sum *= gate_value(g, a.gate_act);
         }
         return sum;
+    };
+    auto late_gate = [&](int c) {                          // the gate of column c of the whole row, where it follows the norm
+        if (a.gate == nullptr || !a.gate_after_norm) return 1.f;
+        return gate_value(load_as_float(a.gate, a.gate_is_float32 ? XRT_F32 : dtype, row * a.gate_stride + c), a.gate_act);
     };
     auto gated = [&](int c) {
         float sum = raw[out_at + c];
@@ -461,11 +473,17 @@ __global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kerne
             kept[i] = fmaf(load_as_float(a.skip, a.skip_dtype, (c0 + c) / a.vdim), values[i], kept[i]);
         }
     }
+    float gates[FINISH_KEPT];
+#pragma unroll
+    for (int i = 0; i < FINISH_KEPT; ++i) gates[i] = 1.f;
     if (a.gate != nullptr) {
-        float gates[FINISH_KEPT];
         load_kept(a.gate, a.gate_is_float32 || dtype == XRT_F32, row * a.gate_stride + c0, 1, gates);
 #pragma unroll
-        for (int i = 0; i < FINISH_KEPT; ++i) kept[i] *= a.gate_act == XRT_GATE_SILU ? silu_exact(gates[i]) : gates[i];
+        for (int i = 0; i < FINISH_KEPT; ++i) gates[i] = gate_value(gates[i], a.gate_act);
+        if (!a.gate_after_norm) {
+#pragma unroll
+            for (int i = 0; i < FINISH_KEPT; ++i) { kept[i] *= gates[i]; gates[i] = 1.f; }
+        }
     }
 #pragma unroll
     for (int i = 0; i < FINISH_KEPT; ++i) {
@@ -482,12 +500,12 @@ __global__ void __launch_bounds__(FINISH_THREADS) recurrence_finish_groups_kerne
 #pragma unroll
     for (int i = 0; i < FINISH_KEPT; ++i) {
         const int c = threadIdx.x + i * FINISH_THREADS;
-        if (c < part_width) store_from_float(a.out, dtype, out_at + c0 + c, kept[i] * inv * weights[i]);
+        if (c < part_width) store_from_float(a.out, dtype, out_at + c0 + c, kept[i] * inv * weights[i] * gates[i]);
     }
     for (int c = threadIdx.x + FINISH_KEPT * FINISH_THREADS; c < part_width; c += FINISH_THREADS) {
         float value = gated(c0 + c) * inv;
         if (a.norm_weight != nullptr) value *= load_as_float(a.norm_weight, a.norm_weight_dtype, c0 + c);
-        store_from_float(a.out, dtype, out_at + c0 + c, value);
+        store_from_float(a.out, dtype, out_at + c0 + c, value * late_gate(c0 + c));
     }
 }
 
@@ -628,6 +646,9 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
                 "linear_recurrence: unknown decay mode %d, or no decays", a.decay_mode);
     XRT_REQUIRE(a.decay_mode != XRT_DECAY_STEP || (a.decay_rate != nullptr && a.decay_stride >= a.heads),
                 "linear_recurrence: decays from step sizes need a rate per head and the steps' row stride");
+    XRT_REQUIRE(!a.input_silu || (a.bonus == nullptr && a.skip == nullptr), "linear_recurrence: activated inputs go with neither a bonus nor a skip");
+    XRT_REQUIRE(!a.gate_after_norm || a.norm_groups > 0, "linear_recurrence: a gate after the norm goes with a norm over parts of the whole row");
+    XRT_REQUIRE(a.gate_act >= XRT_GATE_PLAIN && a.gate_act <= XRT_GATE_SIGMOID, "linear_recurrence: unknown gate activation %d", a.gate_act);
     XRT_REQUIRE(a.qk_heads == 0 || (a.qk_heads > 0 && a.heads % a.qk_heads == 0), "linear_recurrence: %d heads cannot share %d heads of q and k", a.heads, a.qk_heads);
     XRT_REQUIRE(a.norm_groups == 0 || (a.norm != 0 && a.norm_groups > 0 && (a.heads * a.vdim) % a.norm_groups == 0 && a.norm_groups <= 65535 &&
                                        (a.norm_weight == nullptr || a.norm_weight_per_head || a.heads == 1)),

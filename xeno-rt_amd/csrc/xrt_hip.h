@@ -220,7 +220,7 @@ int xrt_short_conv(const void* x, int dtype, long tokens, long x_stride, int cha
 // square of each of its norm_groups equal parts, times norm_weight [heads * vdim]. gate_is_float32: the gate's rows are float32
 // whatever the element type.
 enum { XRT_DECAY_PER_HEAD = 0, XRT_DECAY_GIVEN = 1, XRT_DECAY_EXP_NEG_EXP = 2, XRT_DECAY_SIGMOID_POWER = 3, XRT_DECAY_STEP = 4 };
-enum { XRT_GATE_PLAIN = 0, XRT_GATE_SILU = 1 };
+enum { XRT_GATE_PLAIN = 0, XRT_GATE_SILU = 1, XRT_GATE_SIGMOID = 2 };
 typedef struct {
     const void *q, *k, *v;
     long q_stride, k_stride, v_stride;
@@ -250,6 +250,8 @@ typedef struct {
     int skip_dtype;
     int norm_groups;
     int gate_is_float32;
+    int input_silu;          // q, k and v are silu of what the pointers hold
+    int gate_after_norm;     // with norm_groups: norm and weight first, then the gate
 } xrt_recurrence;
 // token_slots [tokens]: the slot of every token's sequence. The workspace holds the raw outputs and, where a long prompt is cut
 // into segments that run side by side, the segments' states; xrt_linear_recurrence_workspace says how many floats.
@@ -274,7 +276,8 @@ int xrt_kv_store(const void* k, long k_stride, const void* v, long v_stride, int
                  int value_dim, const int* positions, const int* slots, void* k_cache, void* v_cache, const int* block_table,
                  int table_stride, int n_blocks, void* stream);
 
-// The general attention kernel with values of a width of their own and, with sink, one more key of score 0 that has no value.
+// The general attention kernel with values of a width of their own and, with sink, one more key that has no value: its score is 0,
+// or, with sink_scores (float32 [n_heads]), the head's own number, which is neither scaled nor biased.
 // q_stride: 0 (rows of qkv are q, k and v side by side), or the distance between the rows of q where they lie alone (keys and
 // values are read from the cache only). distance_bias: null, or float32 [n_heads][bias_span]: a key d tokens behind the query
 // adds distance_bias[h][min(d, bias_span - 1)] to its scaled score (any bias that is a function of head and distance and
@@ -283,8 +286,8 @@ int xrt_kv_store(const void* k, long k_stride, const void* v, long v_stride, int
 int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* positions, const int* slots, void* out, float scale, int window,
-                          const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
-                          int chunk, void* stream);
+                          const float* distance_slopes, int sink, const float* sink_scores, long q_stride, const float* distance_bias,
+                          int bias_span, int chunk, void* stream);
 
 // The matrix-core attention for a step that brings sequences of many tokens, with the queries alone in q (rows q_stride
 // apart; keys and values are in the cache) and, with chunk > 0, queries that see the keys of their own stretch of `chunk`
@@ -318,13 +321,16 @@ int xrt_attention_sigmoid(const void* q, long q_stride, int dtype, long tokens, 
 // and sines times magnitude); values_out (or null) takes the values as projected (float32 [tokens][n_kv_heads * value_dim]);
 // with values_in (same shape, or null) v <- (1 - lambda) v + lambda values_in, lambda one number on the device; q goes to
 // q_out (element type `dtype`, rows q_stride apart), k and v into the cache (or nowhere, if the caches are null). Biases, norm
-// weights and lambda have the element type small_dtype.
+// weights and lambda have the element type small_dtype. plain_norm: the head norm without a gain (norm_q and norm_k null).
+// temp_every > 0: the queries of the token at position p are multiplied by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1).
+// queries_only: the rows of proj hold [q heads | anything] and nothing is written but q_out.
 int xrt_qkv_complete(const float* proj, long proj_stride, int dtype, long tokens, int n_heads, int n_kv_heads, int head_dim,
                    int value_dim, const void* bias_q, const void* bias_k, const void* bias_v, const void* norm_q,
                    const void* norm_k, float norm_eps, int small_dtype, const float* frequencies, int rot_dims,
                    int neighbours, float magnitude, const float* values_in, float* values_out, const void* lambda,
                    const int* positions, const int* slots, void* q_out, long q_stride, void* k_cache, void* v_cache,
-                   const int* block_table, int table_stride, int n_blocks, void* stream);
+                   const int* block_table, int table_stride, int n_blocks, int plain_norm, float temp_coef, int temp_every,
+                   int queries_only, void* stream);
 
 // Layer norm of whole rows, y = (x - mean) / sqrt(mean of squared deviations + eps) * weight + bias; x float32, weight and
 // bias of w_dtype. xrt_layernorm: out[r] = norm(x[rows ? rows[r] : r]).
@@ -391,9 +397,10 @@ int xrt_cast(const void* x, int x_dtype, void* out, int out_dtype, long count, v
 // groups of neighbours, a group's score the sum of its group_top largest scores, experts of the `keep` best groups stay
 // open; the `top` largest open scores are chosen; weights [tokens][experts] (float32) get score / (sum of the chosen scores
 // + floor) for the chosen and 0 for the others; chosen (or null) [tokens][top] the experts in the order of their scores.
+// softmax != 0: the scores are softmax(z) over all experts instead; scale multiplies the chosen experts' weights.
 #define XRT_MOST_EXPERTS 256
 int xrt_route_experts(const float* logits, long tokens, int experts, int top, int groups, int keep, int group_top, float floor_,
-                      float* weights, int* chosen, void* stream);
+                      float* weights, int* chosen, int softmax, float scale, void* stream);
 // act[t][e * width + c] *= weights[t][e]
 int xrt_scale_blocks(void* act, int dtype, const float* weights, long tokens, int experts, int width, void* stream);
 
@@ -417,6 +424,35 @@ int xrt_linear_groups(const void* a, int lda, const void* w, long w_stride, int 
                       int tile, long tiles, int n, int k, int coded_mode, const int* tile_group, int parts, void* stream);
 int xrt_experts_combine(const float* sorted, const int* places, const int* chosen, const float* weights, long tokens, int top, int experts,
                         int width, int tile, int parts, float* out, void* stream);
+
+// ---- a residual stream in several copies (csrc/streams.hip) ------------------------------------------------------------------
+// streams: float32 [tokens][copies][width]. open: every copy is the token's row of x. read: out[r] = norm(sum over the copies s
+// of in[s] * copy s of token rows[r] (or r)), the norm being u / sqrt(mean(u^2) + eps) * gain, or u itself with a null gain.
+// write: all copies at once from the old ones, copy t <- sum over s of mix[s][t] * copy s + out_weights[t] * y (y float32
+// [tokens][width]); with next_in the read of the new copies under next_in, gain and eps goes to `normed` in the same pass.
+// in, mix and out_weights are float32 on the device.
+#define XRT_MOST_STREAMS 8
+int xrt_streams_open(const float* x, float* streams, long tokens, int width, int copies, void* stream);
+int xrt_streams_read(const float* streams, int copies, const float* in, const void* gain, int gain_dtype, float eps, void* out,
+                     int out_dtype, const int* rows, long n_rows, int width, void* stream);
+int xrt_streams_write(float* streams, int copies, const float* mix, const float* out_weights, const float* y, long tokens, int width,
+                      const float* next_in, const void* gain, int gain_dtype, float eps, void* normed, int normed_dtype, void* stream);
+
+// ---- attention through a latent (csrc/latent.hip) ---------------------------------------------------------------------------
+// The cache of such a layer has one key/value head whose keys are [latent (rank) | turned key part (rot_dim)] and whose values
+// are the latent. complete: from float32 rows [latent | key part] (down_stride apart) the latent / rms(latent) * gain and the
+// key part with its first rot_dims turned in pairs of neighbours by position * frequencies[pair], into the cache.
+// queries: from float32 rows of heads x [plain (dim) | part to turn (rot_dim)] the plain parts to `plain` [tokens][heads][dim]
+// and the turned parts to full[t][h][rank ..], rows full_stride apart, heads rank + rot_dim apart.
+// linear_heads: out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k]; rows of a and out a_stride and out_stride apart, heads
+// a_head and out_head apart; all three of `dtype`, float32 sums in the order of k.
+int xrt_latent_complete(const float* down, long down_stride, int dtype, long tokens, int rank, int rot_dim, int rot_dims,
+                        const void* gain, int gain_dtype, float eps, const float* frequencies, const int* positions, const int* slots,
+                        void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks, void* stream);
+int xrt_latent_queries(const float* q, long q_stride, int dtype, long tokens, int heads, int dim, int rot_dim, int rot_dims,
+                       const float* frequencies, const int* positions, void* plain, void* full, long full_stride, int rank, void* stream);
+int xrt_linear_heads(const void* a, long a_stride, long a_head, const void* w, int dtype, void* out, long out_stride, long out_head,
+                     long rows, int heads, int n, int k, void* stream);
 
 #ifdef __cplusplus
 }

@@ -32,6 +32,7 @@ class ModelSpec:
     final_norm: Norm
     head: OutputHead
     schedule: Optional[List[LayerCall]] = None
+    streams: Optional[object] = None        # a residual stream in several copies (parts/block.py: ResidualStreams), or None for one
 
     def __post_init__(self):
         if self.schedule is None:
@@ -53,7 +54,7 @@ class ModelSpec:
                                      "whose layer keeps something else")
 
     def parts(self):
-        return [self.embedding, *self.layers, self.final_norm, self.head]
+        return [self.embedding, *self.layers, self.final_norm, self.head] + ([self.streams] if self.streams is not None else [])
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         specs: Dict[str, WeightSpec] = {}
@@ -106,6 +107,8 @@ class DecoderModel:
             x = spec.embedding.forward_step(batch, cache.layer_cache(len(spec.schedule)))
         else:
             x = spec.embedding.forward(batch.token_ids, batch.positions)
+        if spec.streams is not None:                             # the blocks then work on the copies [tokens, copies, hidden]
+            x = spec.streams.open(x)
         h = None            # the next block's first norm of x, where the block before it has made it already
         for index, call in enumerate(spec.schedule):
             block = spec.layers[call.layer]
@@ -118,5 +121,8 @@ class DecoderModel:
             h = block.forward(x, batch, cache.layer_cache(index), h=h, then=then)
         if batch.n_logit_rows == 0:
             return self.runtime.empty((0, spec.head.vocab), torch.float32, outlives_the_step=True)
-        y = spec.final_norm.forward(x, rows=batch.logit_rows)
+        if spec.streams is not None:
+            y = spec.streams.close(x, spec.final_norm, rows=batch.logit_rows)
+        else:
+            y = spec.final_norm.forward(x, rows=batch.logit_rows)
         return spec.head.forward(y)

@@ -136,7 +136,8 @@ class _Recurrence(ctypes.Structure):
                 ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_long), ("gate_act", ctypes.c_int), ("out", ctypes.c_void_p),
                 ("decay_stride", ctypes.c_long), ("decay_rate", ctypes.c_void_p), ("decay_rate_dtype", ctypes.c_int),
                 ("qk_heads", ctypes.c_int), ("skip", ctypes.c_void_p), ("skip_dtype", ctypes.c_int),
-                ("norm_groups", ctypes.c_int), ("gate_is_float32", ctypes.c_int)]
+                ("norm_groups", ctypes.c_int), ("gate_is_float32", ctypes.c_int), ("input_silu", ctypes.c_int),
+                ("gate_after_norm", ctypes.c_int)]
 
 
 class _SelectiveScan(ctypes.Structure):
@@ -200,7 +201,8 @@ class HipOps:
                      "xrt_bigram_add", "xrt_gated_rows", "xrt_add_weighted", "xrt_glu_clamped", "xrt_softcap", "xrt_cast",
                      "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts",
                      "xrt_experts_sort", "xrt_gather_rows", "xrt_linear_groups", "xrt_linear_groups_accepts", "xrt_experts_combine",
-                     "xrt_linear_groups_tile_rows", "xrt_linear_groups_parts"):
+                     "xrt_linear_groups_tile_rows", "xrt_linear_groups_parts", "xrt_streams_open", "xrt_streams_read", "xrt_streams_write",
+                     "xrt_latent_complete", "xrt_latent_queries", "xrt_linear_heads"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -486,21 +488,22 @@ class HipOps:
                                                         0 if rope_table is None else int(rope_table.shape[0]), int(batch.max_context)))
 
     def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None,
-                  finish: Optional[QkvFinish] = None, value_dim: Optional[int] = None, sink: bool = False,
+                  finish: Optional[QkvFinish] = None, value_dim: Optional[int] = None, sink=False,
                   distance_bias: Optional[torch.Tensor] = None, queries_alone: bool = False, chunk: Optional[int] = None):
         """Causal attention of the step's tokens over the cache. chunk: positions are cut into stretches of this many from a
         sequence's first token on, and a query sees the keys of its own stretch only. distance_slopes: float32 [n_heads], or None; a key at
         position j adds slope * (j - P) to the scaled score of the query at position P. distance_bias: float32
         [n_heads, span], or None; a key d tokens behind the query adds distance_bias[h, min(d, span - 1)]. queries_alone: the
-        rows of `qkv` hold the queries only (keys and values are in the cache already). finish: what is still to do to
+        rows of `qkv` hold the queries only (keys and values are in the cache already). sink: True, or float32 [n_heads]: the softmax's
+        denominator has one more term, exp(0) or exp of the head's number. finish: what is still to do to
         q, k and v (only where `attention_finishes_qkv` says so); the cache must be writable then."""
         from ..cache import BLOCK_TOKENS
         if finish is not None:
             return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
-        if (queries_alone and not sink and distance_bias is None and distance_slopes is None and not window
+        if (queries_alone and sink is False and distance_bias is None and distance_slopes is None and not window
                 and self._attention_stretches(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, chunk)):
             return None
-        if sink or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone or chunk:
+        if sink is not False or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone or chunk:
             return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
                                            distance_slopes, sink, distance_bias, queries_alone, chunk)
         tokens = qkv.shape[0]
@@ -572,7 +575,8 @@ class HipOps:
     def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink,
                            distance_bias=None, queries_alone=False, chunk=None):
         """Rows of qkv are [n_heads x head_dim | n_kv_heads x head_dim | n_kv_heads x value_dim] (or the queries alone), rows of
-        out n_heads x value_dim. sink: the softmax's denominator has one more (a key of score 0 without a value)."""
+        out n_heads x value_dim. sink: the softmax's denominator has one more (a key without a value whose score is 0 or, if sink is
+        a tensor float32 [n_heads], the head's number there)."""
         tokens = qkv.shape[0]
         q_stride = 0
         if queries_alone:
@@ -589,10 +593,13 @@ class HipOps:
         k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim, value_dim)
         if distance_slopes is not None:
             self._require(distance_slopes, "attention distance_slopes", torch.float32, (n_heads,), qkv)
+        sink_scores = sink if isinstance(sink, torch.Tensor) else None
+        if sink_scores is not None:
+            self._require(sink_scores, "attention sink", torch.float32, (n_heads,), qkv)
         self._check(self.lib.xrt_attention_general(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, value_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table), stride,
             n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale), int(window or 0),
-            _ptr(distance_slopes), int(bool(sink)), ctypes.c_long(q_stride), _ptr(distance_bias), int(span), int(chunk or 0),
+            _ptr(distance_slopes), int(sink is not False and sink is not None), _ptr(sink_scores), ctypes.c_long(q_stride), _ptr(distance_bias), int(span), int(chunk or 0),
             self._stream(qkv)))
 
     def attention_sigmoid(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window=None, head_mix=None,
@@ -628,15 +635,18 @@ class HipOps:
 
     def qkv_complete(self, proj, n_heads, n_kv_heads, head_dim, value_dim, batch, q_out, kv=None, biases=None, norms=None,
                      norm_eps=0.0, frequencies=None, rot_dims=0, neighbours=True, magnitude=1.0, values_in=None, values_out=None,
-                     blend=None):
+                     blend=None, plain_norm=False, query_temperature=None, queries_only=False):
         """What lies between an attention's projection and its scores. proj: float32 rows [q | k | v | ...] (the leading columns
         of the projection's output). biases: (q, k, v) vectors or None; norms: (q, k) weights [head_dim] of an RMS norm of every
         head, or None; frequencies: float32 [rot_dims / 2], the first rot_dims dims of every head of q and k turn by
         position * frequency in pairs of neighbours (or of halves), cosines and sines times magnitude; values_out: float32
         [tokens, n_kv_heads * value_dim] takes the values as projected; values_in (same shape) with blend (one number on the
-        device): v <- (1 - blend) v + blend values_in. q goes to q_out (compute dtype), k and v into the cache `kv` (if given)."""
+        device): v <- (1 - blend) v + blend values_in. q goes to q_out (compute dtype), k and v into the cache `kv` (if given).
+        plain_norm: every head of q and k is divided by its root mean square (no weights). query_temperature = (coef, every): the
+        queries at position p times 1 + coef * ln(floor((p + 1) / every) + 1). queries_only: proj holds [q | ...] and only q_out
+        is written (biases = (q's, None, None))."""
         tokens = proj.shape[0]
-        width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
+        width = n_heads * head_dim if queries_only else (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
         if proj.dim() != 2 or proj.shape[1] < width:
             raise KernelError(f"qkv_complete proj: {tuple(proj.shape)}, expected at least {width} columns")
         proj_stride = self._rows(proj, "qkv_complete proj", None, torch.float32)
@@ -649,8 +659,9 @@ class HipOps:
         if biases is not None:
             b_q, b_k, b_v = biases
             self._require(b_q, "qkv_complete bias of q", small_dtype, (n_heads * head_dim,), proj)
-            self._require(b_k, "qkv_complete bias of k", small_dtype, (n_kv_heads * head_dim,), proj)
-            self._require(b_v, "qkv_complete bias of v", small_dtype, (n_kv_heads * value_dim,), proj)
+            if not queries_only:
+                self._require(b_k, "qkv_complete bias of k", small_dtype, (n_kv_heads * head_dim,), proj)
+                self._require(b_v, "qkv_complete bias of v", small_dtype, (n_kv_heads * value_dim,), proj)
         if norms is not None:
             n_q, n_k = norms
             self._require(n_q, "qkv_complete norm of q", small_dtype, (head_dim,), proj)
@@ -668,12 +679,13 @@ class HipOps:
         stride = n_blocks = 0
         if kv is not None:
             k_cache, v_cache, table, stride, n_blocks = self._kv(kv, q_out, n_kv_heads, head_dim, value_dim)
+        temp_coef, temp_every = (0.0, 0) if query_temperature is None else (float(query_temperature[0]), int(query_temperature[1]))
         self._check(self.lib.xrt_qkv_complete(
             _ptr(proj), ctypes.c_long(proj_stride), _code(q_out), ctypes.c_long(tokens), n_heads, n_kv_heads, head_dim, value_dim,
             _ptr(b_q), _ptr(b_k), _ptr(b_v), _ptr(n_q), _ptr(n_k), ctypes.c_float(norm_eps), _CODES[small_dtype], _ptr(frequencies),
             int(rot_dims), int(bool(neighbours)), ctypes.c_float(magnitude), _ptr(values_in), _ptr(values_out), _ptr(blend),
             _ptr(batch.positions), _ptr(batch.slots), _ptr(q_out), ctypes.c_long(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(table),
-            stride, n_blocks, self._stream(proj)))
+            stride, n_blocks, int(bool(plain_norm)), ctypes.c_float(temp_coef), temp_every, int(bool(queries_only)), self._stream(proj)))
 
     # -- layer norm ---------------------------------------------------------------------------------
     def layernorm(self, x, weight, bias, eps, out, rows=None):
@@ -795,7 +807,8 @@ class HipOps:
 
     def linear_recurrence(self, q, k, v, state, batch, out, heads, dim, vdim, decay, decay_mode="per_head", decay_bias=None,
                           decay_power=1.0, q_scale=1.0, k_scale=1.0, bonus=None, norm_eps=None, norm_weight=None, gate=None,
-                          gate_activation="silu", decay_rate=None, qk_heads=None, skip=None, norm_groups=None):
+                          gate_activation="silu", decay_rate=None, qk_heads=None, skip=None, norm_groups=None, input_activation=None,
+                          gate_after_norm=False):
         """Per sequence and head S <- diag(decay) S + k v^T, o = S^T q (with `bonus` [heads, dim]: o = (S + diag(bonus) k v^T)^T q
         before the update); state [slots, heads, dim, vdim] float32. decay: float32 [heads] ("per_head") or [tokens, heads * dim]
         ("given": the decay itself; "exp_neg_exp": exp(-exp(z + bias)); "sigmoid_power": sigmoid(z + bias)^decay_power). Then per head
@@ -805,9 +818,15 @@ class HipOps:
         per token and head with decay_bias [heads]; the head's channels all decay by exp(-exp(decay_rate[head]) * step) and v
         enters the state times the step. qk_heads: q and k have this many heads, shared by neighbouring heads in equal groups.
         skip [heads]: o += skip * v. norm_groups: the gate comes before the norm, which then spans each of that many equal
-        parts of the token's whole row, with norm_weight [heads * vdim]."""
+        parts of the token's whole row, with norm_weight [heads * vdim]; gate_after_norm: such a norm and its weight come first and
+        the gate after them. gate_activation: "silu", "sigmoid" or "plain". input_activation "silu": q, k and v are silu of the rows given."""
         tokens = q.shape[0]
         record = _Recurrence()
+        if input_activation not in (None, "silu"):
+            raise KernelError(f"linear_recurrence: input_activation must be None or 'silu', found {input_activation!r}")
+        record.input_silu, record.gate_after_norm = int(input_activation == "silu"), int(bool(gate_after_norm))
+        if gate_after_norm and norm_groups is None:
+            raise KernelError("linear_recurrence: a gate after the norm is served for a norm over parts of the whole row")
         qk = heads if qk_heads is None else int(qk_heads)
         record.qk_heads = qk
         record.q_stride = self._rows(q, "recurrence q", qk * dim)
@@ -854,7 +873,7 @@ class HipOps:
             if gate.dtype not in (q.dtype, torch.float32):
                 raise KernelError(f"recurrence gate: dtype {gate.dtype}, expected {q.dtype} or float32")
             record.gate_is_float32 = int(gate.dtype == torch.float32)
-            record.gate, record.gate_act = gate.data_ptr(), {"plain": 0, "silu": 1}[gate_activation]
+            record.gate, record.gate_act = gate.data_ptr(), {"plain": 0, "silu": 1, "sigmoid": 2}[gate_activation]
         self._require(out, "recurrence out", q.dtype, (tokens, heads * vdim), q)
         record.out = out.data_ptr()
         offsets, slots, n = self._sequences(batch, tokens, q)
@@ -967,9 +986,9 @@ class HipOps:
         self._require(out, "cast out", None, x.shape, x)
         self._check(self.lib.xrt_cast(_ptr(x), _code(x), _ptr(out), _code(out), ctypes.c_long(x.numel()), self._stream(x)))
 
-    def route_experts(self, logits, weights, top, groups=1, keep=1, group_top=2, floor=1e-20, chosen=None):
+    def route_experts(self, logits, weights, top, groups=1, keep=1, group_top=2, floor=1e-20, chosen=None, scores="sigmoid", scale=1.0):
         """From router logits [tokens, experts] (float32) the weights [tokens, experts] (float32; zero for experts not chosen):
-        scores sigmoid(z); experts in `groups` equal groups of neighbours, a group's score the sum of its group_top largest,
+        scores sigmoid(z) or, scores="softmax", softmax(z) over all experts; the chosen weights times `scale` in the end; experts in `groups` equal groups of neighbours, a group's score the sum of its group_top largest,
         experts of the `keep` best groups stay open; the `top` largest open scores are chosen and divided by their sum + floor.
         chosen (int32 [tokens, top], or None) takes the chosen experts in the order of their scores."""
         tokens, experts = logits.shape
@@ -977,8 +996,101 @@ class HipOps:
         self._require(weights, "route_experts weights", torch.float32, (tokens, experts), logits)
         if chosen is not None:
             self._require(chosen, "route_experts chosen", torch.int32, (tokens, top), logits)
+        if scores not in ("sigmoid", "softmax"):
+            raise KernelError(f"route_experts: scores are 'sigmoid' or 'softmax', found {scores!r}")
         self._check(self.lib.xrt_route_experts(_ptr(logits), ctypes.c_long(tokens), experts, int(top), int(groups), int(keep), int(group_top),
-                                               ctypes.c_float(floor), _ptr(weights), _ptr(chosen), self._stream(logits)))
+                                               ctypes.c_float(floor), _ptr(weights), _ptr(chosen), int(scores == "softmax"),
+                                               ctypes.c_float(scale), self._stream(logits)))
+
+    # -- a residual stream in several copies -----------------------------------------------------------
+    def streams_open(self, x, streams):
+        """streams [tokens, copies, width] (float32): every copy is the token's row of x [tokens, width] (float32)."""
+        tokens, copies, width = streams.shape
+        self._require(x, "streams_open x", torch.float32, (tokens, width))
+        self._require(streams, "streams_open streams", torch.float32, None, x)
+        self._check(self.lib.xrt_streams_open(_ptr(x), _ptr(streams), ctypes.c_long(tokens), width, copies, self._stream(x)))
+
+    def streams_read(self, streams, weights, gain, eps, out, rows=None):
+        """out[r] = norm(sum over the copies s of weights[s] * streams[rows[r] or r, s]): the norm is u / sqrt(mean(u^2) + eps) * gain,
+        or, gain None, u itself. streams float32 [tokens, copies, width], weights float32 [copies]."""
+        tokens, copies, width = streams.shape
+        n_rows = tokens if rows is None else rows.shape[0]
+        self._require(streams, "streams_read streams", torch.float32)
+        self._require(weights, "streams_read weights", torch.float32, (copies,), streams)
+        self._require(out, "streams_read out", None, (n_rows, width), streams)
+        if gain is not None:
+            self._require(gain, "streams_read gain", None, (width,), streams)
+        if rows is not None:
+            self._require(rows, "streams_read rows", torch.int32, (n_rows,), streams)
+        self._check(self.lib.xrt_streams_read(_ptr(streams), copies, _ptr(weights), _ptr(gain), 0 if gain is None else _code(gain),
+                                              ctypes.c_float(eps), _ptr(out), _code(out), _ptr(rows), ctypes.c_long(n_rows), width,
+                                              self._stream(streams)))
+
+    def streams_write(self, streams, mix, out_weights, y, then=None):
+        """All copies at once from the old ones: copy t <- sum over s of mix[s, t] * copy s + out_weights[t] * y (y float32
+        [tokens, width]). then = (weights, gain, eps, out): the read of the new copies (as `streams_read`) in the same pass."""
+        tokens, copies, width = streams.shape
+        self._require(streams, "streams_write streams", torch.float32)
+        self._require(mix, "streams_write mix", torch.float32, (copies, copies), streams)
+        self._require(out_weights, "streams_write out_weights", torch.float32, (copies,), streams)
+        self._require(y, "streams_write y", torch.float32, (tokens, width), streams)
+        weights = gain = out = None
+        eps = 0.0
+        if then is not None:
+            weights, gain, eps, out = then
+            self._require(weights, "streams_write next weights", torch.float32, (copies,), streams)
+            self._require(out, "streams_write next out", None, (tokens, width), streams)
+            if gain is not None:
+                self._require(gain, "streams_write gain", None, (width,), streams)
+        self._check(self.lib.xrt_streams_write(_ptr(streams), copies, _ptr(mix), _ptr(out_weights), _ptr(y), ctypes.c_long(tokens), width,
+                                               _ptr(weights), _ptr(gain), 0 if gain is None else _code(gain), ctypes.c_float(eps), _ptr(out),
+                                               0 if out is None else _code(out), self._stream(streams)))
+
+    # -- attention through a latent -----------------------------------------------------------------------
+    def latent_complete(self, down, rank, rot_dim, gain, eps, frequencies, rot_dims, kv, batch, like):
+        """From the float32 rows `down` [latent (rank) | key part (rot_dim)] (columns of a wider matrix will do): the latent divided
+        by its root mean square, times gain, and the key part with its first rot_dims turned in pairs of neighbours by
+        position * frequencies[pair], into the cache `kv` of one key/value head (keys rank + rot_dim wide, values rank wide), whose
+        element type is that of `like`."""
+        tokens = down.shape[0]
+        stride = self._rows(down, "latent_complete down", rank + rot_dim, torch.float32)
+        self._require(gain, "latent_complete gain", None, (rank,), down)
+        if rot_dims:
+            self._require(frequencies, "latent_complete frequencies", torch.float32, (rot_dims // 2,), down)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), down)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), down)
+        k_cache, v_cache, table, table_stride, n_blocks = self._kv(kv, like, 1, rank + rot_dim, rank)
+        self._check(self.lib.xrt_latent_complete(_ptr(down), ctypes.c_long(stride), _code(like), ctypes.c_long(tokens), rank, rot_dim, int(rot_dims),
+                                                 _ptr(gain), _code(gain), ctypes.c_float(eps), _ptr(frequencies), _ptr(batch.positions),
+                                                 _ptr(batch.slots), _ptr(k_cache), _ptr(v_cache), _ptr(table), table_stride, n_blocks,
+                                                 self._stream(down)))
+
+    def latent_queries(self, q, heads, dim, rot_dim, frequencies, rot_dims, batch, plain, full, rank):
+        """From the float32 rows q of heads x [plain (dim) | part to turn (rot_dim)]: the plain parts to `plain` [tokens, heads * dim],
+        the turned parts to the last rot_dim columns of every head of `full` [tokens, heads * (rank + rot_dim)]."""
+        tokens = q.shape[0]
+        stride = self._rows(q, "latent_queries q", heads * (dim + rot_dim), torch.float32)
+        self._require(plain, "latent_queries plain", None, (tokens, heads * dim), q)
+        self._require(full, "latent_queries full", plain.dtype, (tokens, heads * (rank + rot_dim)), q)
+        if rot_dims:
+            self._require(frequencies, "latent_queries frequencies", torch.float32, (rot_dims // 2,), q)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), q)
+        self._check(self.lib.xrt_latent_queries(_ptr(q), ctypes.c_long(stride), _code(plain), ctypes.c_long(tokens), heads, dim, rot_dim,
+                                                int(rot_dims), _ptr(frequencies), _ptr(batch.positions), _ptr(plain), _ptr(full),
+                                                ctypes.c_long(heads * (rank + rot_dim)), rank, self._stream(q)))
+
+    def linear_heads(self, a, w, out, out_head=None):
+        """out[t, h, :n] = w[h] a[t, h]: a [tokens, heads * k], w [heads, n, k], out [tokens, heads * out_head] with the head's
+        n outputs at the beginning of its out_head columns (out_head None: n). One element type, float32 sums in the order of k."""
+        heads, n, k = w.shape
+        tokens = a.shape[0]
+        out_head = n if out_head is None else int(out_head)
+        self._require(a, "linear_heads a", None, (tokens, heads * k))
+        self._require(w, "linear_heads w", a.dtype, None, a)
+        self._require(out, "linear_heads out", a.dtype, (tokens, heads * out_head), a)
+        self._check(self.lib.xrt_linear_heads(_ptr(a), ctypes.c_long(heads * k), ctypes.c_long(k), _ptr(w), _code(a), _ptr(out),
+                                              ctypes.c_long(heads * out_head), ctypes.c_long(out_head), ctypes.c_long(tokens), heads, n, k,
+                                              self._stream(a)))
 
     # -- experts that multiply only the tokens that chose them
     def _expert_matrices(self, w_gate_up, w_down, experts, width):

@@ -5,10 +5,11 @@ from .norm import LayerNorm, OffsetRMSNorm, RMSNorm, ScalarRMSNorm
 from .position import DistanceBuckets, DistanceSlopes, NoPosition, PairRotation, Rotary
 from .convolution import ShortConvolution, TokenShift
 from .attention import Attention, SharedValues
-from .recurrent import GatedLinearAttention, Retention, SelectiveStateSpace, StateSpaceDuality, TimeMixWKV
+from .latent import LatentAttention
+from .recurrent import GatedLinearAttention, LightningAttention, Retention, SelectiveStateSpace, StateSpaceDuality, TimeMixWKV
 from .parallel import ParallelMixer, WeightedPair
 from .feedforward import ClampedGLU, DenseMLP, ExpertsMLP, GatedMLP
-from .block import ParallelBlock, PreNormBlock, SandwichBlock
+from .block import HyperConnectionBlock, ParallelBlock, PreNormBlock, ResidualStreams, SandwichBlock
 from .embedding import Embedding, HashedPairEmbedding, OutputHead, PositionedEmbedding, TokenSideInput, TokenSideTable
 
 __all__ = [
@@ -18,5 +19,6 @@ __all__ = [
     "ScalarRMSNorm", "DistanceSlopes", "ShortConvolution", "TokenShift", "GatedLinearAttention", "Retention", "TimeMixWKV",
     "ParallelMixer", "DenseMLP", "PositionedEmbedding", "LayerNorm", "DistanceBuckets", "PairRotation", "SharedValues",
     "SandwichBlock", "OffsetRMSNorm", "SelectiveStateSpace", "StateSpaceDuality", "WeightedPair", "ClampedGLU", "ExpertsMLP",
-    "ParallelBlock", "HashedPairEmbedding", "TokenSideInput", "TokenSideTable",
+    "ParallelBlock", "HashedPairEmbedding", "TokenSideInput", "TokenSideTable", "HyperConnectionBlock", "ResidualStreams",
+    "LatentAttention", "LightningAttention",
 ]

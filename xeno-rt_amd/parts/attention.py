@@ -30,7 +30,12 @@ attention layer made of the same token, v <- (1 - lambda) v + lambda v_other (`v
 layer whose values are kept for the step, `.reader(name)` in those that blend them in, lambda the tensor `name`); a
 position encoding that says `pair_rotation()`, or one that says `score_bias_table()`; positions cut into stretches of
 `chunk` from a sequence's first token on, a query seeing the keys of its own stretch only; or `completed=True`, which
-asks for this path outright (float32 sums of the projection, whatever else the layer has).
+asks for this path outright (float32 sums of the projection, whatever else the layer has). On this path too: biases on q, k
+and v but not on the output (`biases="qkv"`); head norms without weights (`qk_norm="plain"`: every head of q and k divided by
+its root mean square); a query temperature (`query_temperature=(coef, every)`: the queries at position p times
+1 + coef * ln(floor((p + 1) / every) + 1)); a sink with a learnt score per head (`sink="name"` of the tensor [n_heads]: the
+softmax's denominator also holds exp of it, neither scaled nor biased); and a layer without keys and values of its own
+(`keys_from_another=True`: no k and v tensors; its schedule entry reads the cache entry of the layer whose keys and values it uses).
 """
 from __future__ import annotations
 
@@ -71,17 +76,28 @@ class Attention(Mixer):
                  window: Optional[int] = None, value_dim: Optional[int] = None, sink: bool = False,
                  convolution=None, names: Optional[Dict[str, str]] = None, biases: bool = False, weights: str = "softmax",
                  head_mix: Optional[str] = None, score_bias: Optional[str] = None, output_gate: Optional[str] = None,
-                 values=None, unread=(), chunk: Optional[int] = None, completed: bool = False):
+                 values=None, unread=(), chunk: Optional[int] = None, completed: bool = False, query_temperature=None,
+                 keys_from_another: bool = False):
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
             raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
         if weights not in ("softmax", "sigmoid"):
             raise ValueError(f"the weights of the keys are 'softmax' or 'sigmoid', found {weights!r}")
         if weights == "softmax" and (head_mix is not None or score_bias is not None):
             raise ValueError("a mix of the heads' scores and a number per head belong to sigmoid weights")
+        if biases not in (True, False, "qkv") or qk_norm not in (True, False, "plain"):
+            raise ValueError(f"biases are True, False or 'qkv', head norms True, False or 'plain'; found {biases!r} and {qk_norm!r}")
         self.value_dim = head_dim if value_dim is None else int(value_dim)
+        self.sink_name = sink if isinstance(sink, str) else None     # a learnt score per head; sink=True is a score of 0
         self.sink = bool(sink)
         self.convolution = convolution
         self.biases, self.weights = bool(biases), weights
+        self.output_bias = biases is True
+        self.plain_norm = qk_norm == "plain"
+        qk_norm = qk_norm is True
+        self.query_temperature = None if query_temperature is None else (float(query_temperature[0]), int(query_temperature[1]))
+        if self.query_temperature is not None and self.query_temperature[1] <= 0:
+            raise ValueError(f"a query temperature grows every so many positions, found {query_temperature!r}")
+        self.keys_from_another = bool(keys_from_another)
         self.head_mix_name, self.score_bias_name, self.gate_name = head_mix, score_bias, output_gate
         self.values = values
         self.unread = tuple(unread)         # tensors under the prefix that a checkpoint may carry and this layer does not read
@@ -89,9 +105,14 @@ class Attention(Mixer):
         if self.chunk is not None and (self.chunk <= 0 or weights != "softmax"):
             raise ValueError("stretches of positions have a positive size and are served for softmax weights")
         self.completed = (bool(completed) or self.biases or weights == "sigmoid" or output_gate is not None or values is not None or self.chunk is not None
-                          or hasattr(position, "pair_rotation") or hasattr(position, "score_bias_table"))
-        if self.completed and (self.sink or convolution is not None):
-            raise ValueError("the completed path of attention has neither sink nor convolution")
+                          or hasattr(position, "pair_rotation") or hasattr(position, "score_bias_table") or self.sink_name is not None
+                          or self.plain_norm or self.query_temperature is not None or self.keys_from_another)
+        if self.completed and convolution is not None:
+            raise ValueError("the completed path of attention has no convolution")
+        if self.sink and weights != "softmax":
+            raise ValueError("a sink joins a softmax's denominator")
+        if self.keys_from_another and values is not None:
+            raise ValueError("a layer without values of its own blends none")
         if weights == "sigmoid" and hasattr(position, "score_bias_table"):
             raise ValueError("a bias by distance is served for softmax weights")
         self.general = self.completed or self.sink or self.value_dim != head_dim or convolution is not None
@@ -123,12 +144,13 @@ class Attention(Mixer):
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         p, n = self.prefix, self.names
-        specs = {
-            p + n["q"]: WeightSpec((self.q_width, self.hidden)),
-            p + n["k"]: WeightSpec((self.kv_width, self.hidden)),
-            p + n["v"]: WeightSpec((self.v_width, self.hidden)),
-            p + n["o"]: WeightSpec((self.hidden, self.n_heads * self.value_dim)),
-        }
+        specs = {p + n["q"]: WeightSpec((self.q_width, self.hidden)),
+                 p + n["o"]: WeightSpec((self.hidden, self.n_heads * self.value_dim))}
+        if not self.keys_from_another:
+            specs[p + n["k"]] = WeightSpec((self.kv_width, self.hidden))
+            specs[p + n["v"]] = WeightSpec((self.v_width, self.hidden))
+        if self.sink_name is not None:
+            specs[p + self.sink_name] = WeightSpec((self.n_heads,), init="zeros", kind="vector")
         if self.qk_norm:
             specs[p + n["q_norm"]] = WeightSpec((self.head_dim,), init="ones", kind="vector")
             specs[p + n["k_norm"]] = WeightSpec((self.head_dim,), init="ones", kind="vector")
@@ -136,6 +158,8 @@ class Attention(Mixer):
             specs.update(self.convolution.weight_specs())
         if self.biases:
             for name, width in (("q", self.q_width), ("k", self.kv_width), ("v", self.v_width), ("o", self.hidden)):
+                if (name == "o" and not self.output_bias) or (name in "kv" and self.keys_from_another):
+                    continue
                 specs[p + n[name + "_bias"]] = WeightSpec((width,), init="zeros", kind="vector")
         if self.head_mix_name is not None:
             specs[p + self.head_mix_name] = WeightSpec((self.n_heads, self.n_heads), kind="vector")
@@ -151,7 +175,7 @@ class Attention(Mixer):
 
     @property
     def has_output_bias(self) -> bool:
-        return self.biases
+        return self.output_bias
 
     def ignored_names(self):
         """Tensors that a checkpoint may carry for this layer and that it does not read (the share of a blend in a layer
@@ -169,13 +193,17 @@ class Attention(Mixer):
         if self.position is not None:
             self.position.bind(tensors, runtime)
         if self.completed:
-            self.w_proj = runtime.weight([tensors[p + n[name]] for name in "qkv"]
+            projected = "q" if self.keys_from_another else "qkv"
+            self.w_proj = runtime.weight([tensors[p + n[name]] for name in projected]
                                          + ([tensors[p + self.gate_name]] if self.gate_name is not None else []))
             self.w_o = runtime.weight(tensors[p + n["o"]])
-            self.bias_qkv = self.bias_o = self.head_norms = self.head_mix = self.score_bias = self.blend = None
+            self.bias_qkv = self.bias_o = self.head_norms = self.head_mix = self.score_bias = self.blend = self.sink_scores = None
             if self.biases:
-                self.bias_qkv = tuple(runtime.vector(tensors[p + n[name + "_bias"]]) for name in "qkv")
-                self.bias_o = runtime.vector(tensors[p + n["o_bias"]])
+                self.bias_qkv = tuple(runtime.vector(tensors[p + n[name + "_bias"]]) if name in projected else None for name in "qkv")
+                if self.output_bias:
+                    self.bias_o = runtime.vector(tensors[p + n["o_bias"]])
+            if self.sink_name is not None:
+                self.sink_scores = tensors[p + self.sink_name].to(device=runtime.device, dtype=torch.float32).contiguous()
             if self.qk_norm:
                 self.head_norms = (runtime.vector(tensors[p + n["q_norm"]]), runtime.vector(tensors[p + n["k_norm"]]))
             if self.head_mix_name is not None:
@@ -228,7 +256,7 @@ class Attention(Mixer):
         rt = self.runtime
         ops = rt.ops
         tokens = h.shape[0]
-        qkv_width = self.q_width + self.kv_width + self.v_width
+        qkv_width = self.q_width if self.keys_from_another else self.q_width + self.kv_width + self.v_width
         proj = rt.empty((tokens, qkv_width + (self.n_heads if self.gate_name is not None else 0)), torch.float32)
         ops.linear(h, self.w_proj, proj)
         rotation = self.position.pair_rotation() if hasattr(self.position, "pair_rotation") else (None, 0, True, 1.0)
@@ -243,9 +271,10 @@ class Attention(Mixer):
                     raise ValueError("the values to blend in are those of an earlier layer of this step, of the same width")
         q = rt.empty((tokens, self.q_width))
         ops.qkv_complete(proj, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, batch, q,
-                         kv=cache.kv if cache.writable else None, biases=self.bias_qkv, norms=self.head_norms,
-                         norm_eps=self.qk_norm_eps, frequencies=rotation[0], rot_dims=rotation[1], neighbours=rotation[2],
-                         magnitude=rotation[3], values_in=values_in, values_out=values_out, blend=self.blend)
+                         kv=cache.kv if cache.writable and not self.keys_from_another else None, biases=self.bias_qkv,
+                         norms=self.head_norms, norm_eps=self.qk_norm_eps, frequencies=rotation[0], rot_dims=rotation[1],
+                         neighbours=rotation[2], magnitude=rotation[3], values_in=values_in, values_out=values_out, blend=self.blend,
+                         plain_norm=self.plain_norm, query_temperature=self.query_temperature, queries_only=self.keys_from_another)
         out = rt.empty((tokens, self.n_heads * self.value_dim))
         if self.weights == "sigmoid":
             ops.attention_sigmoid(q, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, cache.kv, batch, out, self.scale,
@@ -257,7 +286,8 @@ class Attention(Mixer):
         table = self.position.score_bias_table() if hasattr(self.position, "score_bias_table") else None
         slopes = None if self.position is None else self.position.score_slopes()
         ops.attention(q, self.n_heads, self.n_kv_heads, self.head_dim, cache.kv, batch, out, scale=self.scale, window=self.window,
-                      distance_slopes=slopes, value_dim=self.value_dim, distance_bias=table, queries_alone=True, chunk=self.chunk)
+                      distance_slopes=slopes, value_dim=self.value_dim, distance_bias=table, queries_alone=True, chunk=self.chunk,
+                      sink=self.sink_scores if self.sink_scores is not None else self.sink)
         return out
 
     def forward_into(self, h, batch, cache, out: torch.Tensor, bias_later: bool = False):

@@ -10,11 +10,11 @@ transform per sublayer, a part that is applied to the normed rows before the mix
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
-from .base import Block, CacheNeeds, Runtime, WeightSpec, register_part
+from .base import Block, CacheNeeds, Part, Runtime, WeightSpec, register_part
 
 
 class PreNormBlock(Block):
@@ -220,6 +220,129 @@ class ParallelBlock(Block):
             self.after.forward(x, batch, reads=reads)
 
 
+class ResidualStreams(Part):
+    """The residual stream in `count` copies (hyper-connections): x [tokens, count, width], float32. All copies start as the
+    embedding's rows (`open`); blocks read weighted sums of the copies and write all copies at once (`HyperConnectionBlock`);
+    in the end the copies are added up and normed for the output head (`close`)."""
+    capturable = True
+
+    def __init__(self, count: int, width: int):
+        if count <= 0:
+            raise ValueError(f"a residual stream has one copy at least, found {count}")
+        self.count, self.width = int(count), int(width)
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.ones = torch.ones(self.count, dtype=torch.float32, device=runtime.device)
+
+    def open(self, x: torch.Tensor) -> torch.Tensor:
+        streams = self.runtime.empty((x.shape[0], self.count, self.width), torch.float32)
+        self.runtime.ops.streams_open(x, streams)
+        return streams
+
+    def close(self, streams: torch.Tensor, norm, rows=None) -> torch.Tensor:
+        """norm(sum of the copies) of the tokens in `rows` (all, if None), in the compute dtype."""
+        scale = norm.row_scale()
+        if scale is None:
+            raise ValueError("the norm behind a residual stream in copies is a plain RMS norm")
+        out = self.runtime.empty((streams.shape[0] if rows is None else rows.shape[0], self.width))
+        self.runtime.ops.streams_read(streams, self.ones, scale[0], scale[1], out, rows=rows)
+        return out
+
+
+class _StreamsRead:
+    """What a block's first sublayer reads of the copies: the weights of the sum and the norm behind it."""
+
+    def __init__(self, block):
+        self.block = block
+
+    def arguments(self, out):
+        gain, eps = self.block.mixer_norm.row_scale()
+        return self.block.weights[0]["in"], gain, eps, out
+
+
+class HyperConnectionBlock(Block):
+    """A pre-norm block on a residual stream in copies x_1 .. x_s. For each sublayer (the mixer, then the feed-forward if the
+    block has one) with its three tensors `in` [s], `out` [s] and `mix` [s, s] (from, to): u = sum_s in[s] x_s,
+    y = sublayer(norm(u)), then all copies at once from the old ones, x_t <- sum_s mix[s, t] x_s + out[t] y. The sublayers
+    write their float32 output aside (`forward_into`); one kernel writes the copies and makes the next sublayer's read and
+    norm in the same pass, across blocks too. Norms are plain RMS norms (`row_scale`)."""
+    passes_norms = True
+
+    def __init__(self, count: int, hidden: int, mixer_norm, mixer, mixer_connection: str, feed_forward_norm=None, feed_forward=None,
+                 feed_forward_connection: Optional[str] = None):
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        if feed_forward is not None and feed_forward_connection is None:
+            raise ValueError("a feed-forward on a stream in copies needs its connection's tensors")
+        self.count, self.hidden = int(count), int(hidden)
+        self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward = mixer_norm, mixer, feed_forward_norm, feed_forward
+        self.connections = [mixer_connection] + ([feed_forward_connection] if feed_forward is not None else [])
+        self.weights = []
+
+    def parts(self):
+        return tuple(part for part in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward) if part is not None)
+
+    @property
+    def capturable(self) -> bool:
+        return all(part.capturable for part in self.parts())
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        specs: Dict[str, WeightSpec] = {}
+        for prefix in self.connections:
+            specs[prefix + "in"] = WeightSpec((self.count,), init="ones", kind="vector")
+            specs[prefix + "out"] = WeightSpec((self.count,), init="ones", kind="vector")
+            specs[prefix + "mix"] = WeightSpec((self.count, self.count), init="normal", kind="vector")
+        for part in self.parts():
+            specs.update(part.weight_specs())
+        return specs
+
+    def ignored_names(self):
+        return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
+
+    def cache_needs(self) -> CacheNeeds:
+        return self.mixer.cache_needs()
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        for part in self.parts():
+            part.bind(tensors, runtime)
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and norm.row_scale() is None:
+                raise ValueError("the norms of a block on a stream in copies are plain RMS norms")
+        # (float32 whatever the file stores: the sums over the copies are float32)
+        self.weights = [{name: tensors[prefix + name].to(device=runtime.device, dtype=torch.float32).contiguous()
+                         for name in ("in", "out", "mix")} for prefix in self.connections]
+
+    def first_norm(self):
+        return _StreamsRead(self)
+
+    def forward(self, x, batch, cache, h=None, then=None):
+        """x: the copies [tokens, count, hidden]. h: this block's first read, if the block before has made it; then: the next
+        block's `first_norm()`, whose read this block's last write makes as well (returned; None without `then`)."""
+        rt = self.runtime
+        tokens = x.shape[0]
+        if h is None:
+            h = rt.empty((tokens, self.hidden))
+            weights, gain, eps, _ = _StreamsRead(self).arguments(None)
+            rt.ops.streams_read(x, weights, gain, eps, h)
+        y = rt.empty((tokens, self.hidden), torch.float32)
+        self.mixer.forward_into(h, batch, cache, y)
+        after = None if then is None else then.arguments(rt.empty((tokens, self.hidden)))
+        first = self.weights[0]
+        if self.feed_forward is None:
+            rt.ops.streams_write(x, first["mix"], first["out"], y, then=after)
+            return None if after is None else after[3]
+        second = self.weights[1]
+        gain, eps = self.feed_forward_norm.row_scale()
+        h = rt.empty((tokens, self.hidden))
+        rt.ops.streams_write(x, first["mix"], first["out"], y, then=(second["in"], gain, eps, h))
+        self.feed_forward.forward_into(h, batch, y)
+        rt.ops.streams_write(x, second["mix"], second["out"], y, then=after)
+        return None if after is None else after[3]
+
+
+register_part("block", "hyper_connection", HyperConnectionBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "sandwich", SandwichBlock)

@@ -151,15 +151,29 @@ class ExpertsMLP(FeedForward):
     every token with every expert (the step reads all weights once either way), weights each expert's stretch of the
     activations by the router's weight (zero for experts not chosen) and lets the down product add them up. A step of many
     tokens sorts its picks by expert, and every expert multiplies the rows that chose it (`ops.experts_sorted`). Either way
-    a token's result never depends on what else the step holds."""
+    a token's result never depends on what else the step holds.
+
+    Options: `scores="softmax"` takes the softmax of the logits over all experts as scores; `group_top` is the number of a
+    group's largest scores whose sum is the group's score (1: its largest score); `scale` multiplies the chosen experts'
+    weights; `clamp=(limit, alpha)` makes the experts clamped ones, W_down (g sigmoid(alpha g) (u + 1)) with
+    g = min(W_gate h, limit) and u = clamp(W_up h, -limit, limit): their gate and up rows then lie expert after expert in one
+    matrix whose product keeps float32 sums, which the clamps and the activation read and round once."""
     capturable = True
     GROUP_TOP = 2
     WEIGHT_FLOOR = 1e-20
 
     def __init__(self, prefix: str, hidden: int, intermediate: int, experts: int, top: int, groups=None, keep=None,
-                 router: str = "router", expert: str = "e{}.", gate: str = "gate", up: str = "up", down: str = "down"):
+                 router: str = "router", expert: str = "e{}.", gate: str = "gate", up: str = "up", down: str = "down",
+                 scores: str = "sigmoid", group_top: Optional[int] = None, scale: float = 1.0, clamp=None):
         if experts <= 0 or not 0 < top <= experts:
             raise ValueError(f"{top} of {experts} experts")
+        if scores not in ("sigmoid", "softmax"):
+            raise ValueError(f"the router's scores are 'sigmoid' or 'softmax', found {scores!r}")
+        self.scores, self.scale = scores, float(scale)
+        self.group_top = self.GROUP_TOP if group_top is None else int(group_top)
+        self.clamp = None if clamp is None else (float(clamp[0]), float(clamp[1]))
+        if self.group_top <= 0 or (self.clamp is not None and self.clamp[0] <= 0):
+            raise ValueError("a group's score sums one score at least, and a clamp's limit is positive")
         self.hidden, self.intermediate, self.experts, self.top = hidden, intermediate, int(experts), int(top)
         self.groups, self.keep = (1, 1) if groups is None else (int(groups), int(keep))
         if self.experts % self.groups != 0 or not 0 < self.keep <= self.groups or self.top > self.keep * (self.experts // self.groups):
@@ -179,10 +193,14 @@ class ExpertsMLP(FeedForward):
         super().bind(tensors, runtime)
         self.w_router = runtime.matrix(tensors[self.router_name])
         total = self.experts * self.intermediate
-        # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]; packed for a gated epilogue the
-        # former lies expert after expert, which is what the product of sorted picks reads
-        self.w_gate_up = runtime.weight([tensors[names[0]] for names in self.expert_names] + [tensors[names[1]] for names in self.expert_names],
-                                        "gated", gated_n=total, needed=self.intermediate % 64 == 0 and self.top < self.experts)
+        if self.clamp is not None:
+            # every expert's [gate rows | up rows] one below the other: the float32 sums of a token and an expert are one stretch
+            self.w_gate_up = runtime.weight([tensors[name] for names in self.expert_names for name in names[:2]])
+        else:
+            # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]; packed for a gated epilogue the
+            # former lies expert after expert, which is what the product of sorted picks reads
+            self.w_gate_up = runtime.weight([tensors[names[0]] for names in self.expert_names] + [tensors[names[1]] for names in self.expert_names],
+                                            "gated", gated_n=total, needed=self.intermediate % 64 == 0 and self.top < self.experts)
         down = torch.empty((self.hidden, total), dtype=runtime.dtype, device=runtime.device)
         for n, names in enumerate(self.expert_names):
             down[:, n * self.intermediate:(n + 1) * self.intermediate].copy_(tensors[names[2]])
@@ -193,14 +211,15 @@ class ExpertsMLP(FeedForward):
         logits = rt.empty((h.shape[0], self.experts), torch.float32)
         rt.ops.linear(h, self.w_router, logits)
         weights = rt.empty((h.shape[0], self.experts), torch.float32)
-        rt.ops.route_experts(logits, weights, self.top, self.groups, self.keep, self.GROUP_TOP, self.WEIGHT_FLOOR, chosen=chosen)
+        rt.ops.route_experts(logits, weights, self.top, self.groups, self.keep, self.group_top, self.WEIGHT_FLOOR, chosen=chosen,
+                             scores=self.scores, scale=self.scale)
         return weights
 
     def forward_into(self, h, batch, out: torch.Tensor) -> None:
         rt = self.runtime
         # A step of many tokens of which each uses few of the experts: the picks sorted by expert, every expert multiplies the
         # tokens that chose it. (Where the kernels have no such product, or it would not pay, every token meets every expert.)
-        takes = getattr(rt.ops, "experts_sorted_takes", None)
+        takes = getattr(rt.ops, "experts_sorted_takes", None) if self.clamp is None else None
         if takes is not None and takes(h, self.w_gate_up, self.w_down, self.experts, self.intermediate, self.top):
             chosen = rt.empty((h.shape[0], self.top), torch.int32)
             weights = self._weights(h, chosen)
@@ -208,7 +227,12 @@ class ExpertsMLP(FeedForward):
             return
         weights = self._weights(h)
         act = rt.empty((h.shape[0], self.experts * self.intermediate))
-        rt.ops.linear_glu(h, self.w_gate_up, act, activation="silu")
+        if self.clamp is not None:
+            sums = rt.empty((h.shape[0], 2 * self.experts * self.intermediate), torch.float32)
+            rt.ops.linear(h, self.w_gate_up, sums)
+            rt.ops.glu_clamped(sums.view(-1, 2 * self.intermediate), act.view(-1, self.intermediate), *self.clamp)
+        else:
+            rt.ops.linear_glu(h, self.w_gate_up, act, activation="silu")
         rt.ops.scale_blocks(act, weights, self.intermediate)
         rt.ops.linear(act, self.w_down, out)
 

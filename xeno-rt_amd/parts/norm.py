@@ -20,18 +20,20 @@ from .base import Norm, Runtime, WeightSpec, register_part
 class RMSNorm(Norm):
     capturable = True
 
-    def __init__(self, prefix: str, dim: int, eps: float):
+    def __init__(self, prefix: str, dim: int, eps: float, name: Optional[str] = None):
+        """The gain is the tensor `prefix + "weight"`, or `name` if given."""
         self.prefix = prefix
+        self.name = prefix + "weight" if name is None else name
         self.dim = dim
         self.eps = float(eps)
         self.weight = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {self.prefix + "weight": WeightSpec((self.dim,), init="ones", kind="vector")}
+        return {self.name: WeightSpec((self.dim,), init="ones", kind="vector")}
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        self.weight = runtime.vector(tensors[self.prefix + "weight"])
+        self.weight = runtime.vector(tensors[self.name])
 
     def row_scale(self):
         return self.weight, self.eps

@@ -1,6 +1,6 @@
 """Mixers whose memory is a matrix per head: S <- diag(decay) S + k v^T, read with the query.
 
-Four of them, which differ in where the decay comes from and in what surrounds the recurrence:
+Five of them, which differ in where the decay comes from and in what surrounds the recurrence:
   Retention             a fixed decay per head; k scaled by dim^-1/2; the heads' outputs divided by their root mean
                         square, gated by silu of a projection
   GatedLinearAttention  a decay per key channel and token, sigmoid(z)^(1/tau) with z from a low-rank projection with
@@ -14,6 +14,8 @@ Four of them, which differ in where the decay comes from and in what surrounds t
                         exp(-exp(A_log) step), values enter the state times the step, a skip D per head reads the value
                         itself; queries and keys may be shared by groups of heads; the row of all heads is gated, then
                         RMS-normed in equal parts
+  LightningAttention    a fixed decay per head; q, k and v are silu of their projections and nothing is scaled; the row of
+                        all heads is RMS-normed as one, with a weight, then gated by the sigmoid of a projection
 And one whose memory is a vector per channel (`SelectiveStateSpace`): step sizes per channel from a low-rank projection,
 decays exp(step A) per channel and entry, what is fed and read (B, C) shared by all channels of a token
 (`ops.selective_scan`).
@@ -78,6 +80,47 @@ class Retention(_RecurrentMixer):
         rt.ops.linear_recurrence(qkvg[:, :kd], qkvg[:, kd:2 * kd], qkvg[:, 2 * kd:2 * kd + vd], cache.states[self.state_name], batch, o,
                                  self.heads, self.dim, self.vdim, self.decay, "per_head", k_scale=self.dim ** -0.5,
                                  norm_eps=self.eps, gate=qkvg[:, 2 * kd + vd:], gate_activation="silu")
+        return o
+
+
+class LightningAttention(_RecurrentMixer):
+    """S <- decay_h S + k v^T, o = S^T q per head with q = silu(W_q h), k = silu(W_k h), v = silu(W_v h); the heads' outputs side
+    by side are RMS-normed together with a weight [heads * vdim], multiplied by sigmoid(W_g h), and projected."""
+
+    def __init__(self, prefix: str, hidden: int, heads: int, dim: int, vdim: int, decay: Sequence[float], eps: float,
+                 state_name: str = "lightning"):
+        if len(decay) != heads:
+            raise ValueError(f"lightning attention: {len(decay)} decays for {heads} heads")
+        self.prefix, self.hidden, self.heads, self.dim, self.vdim = prefix, hidden, heads, dim, vdim
+        self.decay_values, self.eps, self.state_name = [float(d) for d in decay], float(eps), state_name
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        p, w, kd, vd = self.prefix, self.hidden, self.heads * self.dim, self.heads * self.vdim
+        return {p + "q": WeightSpec((kd, w)), p + "k": WeightSpec((kd, w)), p + "v": WeightSpec((vd, w)),
+                p + "g": WeightSpec((vd, w)), p + "o": WeightSpec((w, vd)), p + "norm": WeightSpec((vd,), init="ones", kind="vector")}
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(states=((self.state_name, StateSpec((self.heads, self.dim, self.vdim))),))
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        p = self.prefix
+        self.w_in = runtime.weight([tensors[p + name] for name in "qkvg"])
+        self.w_o = runtime.weight(tensors[p + "o"])
+        self.norm_weight = runtime.vector(tensors[p + "norm"])
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float64).to(torch.float32).to(runtime.device)
+
+    def mixed(self, h, batch, cache):
+        rt = self.runtime
+        kd, vd = self.heads * self.dim, self.heads * self.vdim
+        # the activations of q, k, v and the gate are worked out in float32 inside the kernels, from the projection's rows
+        qkvg = rt.empty((h.shape[0], 2 * kd + 2 * vd))
+        rt.ops.linear(h, self.w_in, qkvg)
+        o = rt.empty((h.shape[0], vd))
+        rt.ops.linear_recurrence(qkvg[:, :kd], qkvg[:, kd:2 * kd], qkvg[:, 2 * kd:2 * kd + vd], cache.states[self.state_name], batch, o,
+                                 self.heads, self.dim, self.vdim, self.decay, "per_head", norm_eps=self.eps,
+                                 norm_weight=self.norm_weight, norm_groups=1, gate_after_norm=True, gate=qkvg[:, 2 * kd + vd:],
+                                 gate_activation="sigmoid", input_activation="silu")
         return o
 
 
@@ -291,6 +334,7 @@ class SelectiveStateSpace(_RecurrentMixer):
 
 
 register_part("mixer", "retention", Retention)
+register_part("mixer", "lightning_attention", LightningAttention)
 register_part("mixer", "state_space_duality", StateSpaceDuality)
 register_part("mixer", "selective_state_space", SelectiveStateSpace)
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
