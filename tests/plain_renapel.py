@@ -194,7 +194,9 @@ def under(tensors, prefix):
 
 
 def sublayer(X, connection, norm_weight, eps, run):
-    """One sublayer on the copies: read, norm, run, write."""
+    """One sublayer on the copies: read, norm, run, write. A model without copies has one stream and adds to it."""
+    if connection is None:
+        return X + run(rms_norm(X[0], norm_weight, eps))[None]
     y = run(rms_norm(copies_read(X, connection["in"]), norm_weight, eps))
     return copies_write(X, y, connection["mix"], connection["out"])
 
@@ -203,7 +205,8 @@ def forward(tokens, tensors, config, streams=None):
     """Logits [tokens, vocab] of one whole sequence; `streams`, a list, receives the sum of the copies after every layer."""
     eps = config["norm"]["eps"]
     x = tensors["embed"].to(F)[torch.tensor(list(tokens), dtype=torch.long)]
-    X = x[None].repeat(config.get("streams", 1), 1, 1)
+    copies = config.get("streams")
+    X = x[None].repeat(1 if copies is None else copies, 1, 1)
     kept = {}                   # layer -> its keys and values, for the layers that read them
     for index, layer in enumerate(config["layers"]):
         p = under(tensors, f"l{index}.")
@@ -219,9 +222,10 @@ def forward(tokens, tensors, config, streams=None):
             kept[index] = attention_keys_values(h, mix, m, eps)
             return attention(h, mix, m, eps, kept[index])
 
-        X = sublayer(X, under(p, "hc1."), p["norm1"], eps, mixer)
+        X = sublayer(X, None if copies is None else under(p, "hc1."), p["norm1"], eps, mixer)
         if layer.get("mlp") is not None:
-            X = sublayer(X, under(p, "hc2."), p["norm2"], eps, lambda h: experts_ff(h, under(p, "mlp."), layer["mlp"]))
+            X = sublayer(X, None if copies is None else under(p, "hc2."), p["norm2"], eps,
+                         lambda h: experts_ff(h, under(p, "mlp."), layer["mlp"]))
         if streams is not None:
             streams.append(X.sum(dim=0))
     return rms_norm(X.sum(dim=0), tensors["final.norm"], eps) @ tensors["head"].to(F).T

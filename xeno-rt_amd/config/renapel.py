@@ -6,7 +6,7 @@ a matrix state per head with a fixed decay; `attention`, grouped softmax attenti
 sink, whose keys and values may be another layer's (`kv_from`); `latent_attention`, attention whose keys and values are
 made from a cached latent), the mixer's sizes under `mixer`, and `mlp`: a mixture of experts (`kind` "moe": `expert.ff`,
 `expert.limit`, `router.experts|top|scale|groups.count|groups.keep`) or null. Beside the layers: `vocab`, `width`,
-`norm.eps`, `streams` (the copies of the residual stream). The rows of an attention layer's table of biases are the
+`norm.eps`, `streams` (the copies of the residual stream; absent: one plain residual stream without the copies' weights). The rows of an attention layer's table of biases are the
 table's first dimension; config.json may name them (`bias_rows`) or leave them to the checkpoint.
 """
 from __future__ import annotations
@@ -98,7 +98,7 @@ class RenapelConfig:
     vocab: int
     width: int
     norm_eps: float
-    streams: int
+    streams: Optional[int]                      # None: a plain residual stream
     layers: Tuple[dict, ...]                    # as config.json lists them: {"type", "mixer", "mlp"}
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
@@ -144,12 +144,14 @@ class RenapelConfig:
         eos = () if eos is None else tuple(eos) if isinstance(eos, list) else (eos,)
         return cls(architecture=str(raw.get("architecture") or raw["architectures"][0]), vocab=_positive_int(raw, "vocab"),
                    width=_positive_int(raw, "width"), norm_eps=_number(norm, "eps", "norm"),
-                   streams=_positive_int(raw, "streams") if "streams" in raw else 1, layers=tuple(kept),
+                   streams=_positive_int(raw, "streams") if raw.get("streams") is not None else None, layers=tuple(kept),
                    eos_token_ids=tuple(int(e) for e in eos), bos_token_id=raw.get("bos_token_id"))
 
     def to_dict(self) -> dict:
         out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.norm_eps},
-               "streams": self.streams, "layers": copy.deepcopy(list(self.layers))}
+               "layers": copy.deepcopy(list(self.layers))}
+        if self.streams is not None:
+            out["streams"] = self.streams
         if self.eos_token_ids:
             out["eos_token_id"] = list(self.eos_token_ids)
         if self.bos_token_id is not None:

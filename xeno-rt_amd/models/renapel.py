@@ -1,6 +1,7 @@
 """Renapel: a decoder on a residual stream in several copies, described in parts.
 
-The embedding's rows start every copy of the stream; then the layers that config.json lists, each a block that reads a
+(A configuration without `streams` has one plain residual stream, x += mixer(norm1(x)), x += feed_forward(norm2(x)), and
+no tensors `hc1.*`, `hc2.*`.) The embedding's rows start every copy of the stream; then the layers that config.json lists, each a block that reads a
 weighted sum of the copies before each of its sublayers and writes all copies at once after it
 (parts/block.py: HyperConnectionBlock); in the end the copies are added up, normed, and multiplied by the head. The mixers:
   lightning         a matrix state per head with a fixed decay, q, k and v through silu, the heads' outputs normed together
@@ -19,7 +20,7 @@ from __future__ import annotations
 from ..config import register_architecture
 from ..config.renapel import RenapelConfig
 from ..parts import (Attention, DistanceBuckets, Embedding, ExpertsMLP, HyperConnectionBlock, LatentAttention, LightningAttention,
-                     OutputHead, ResidualStreams, RMSNorm)
+                     OutputHead, PreNormBlock, ResidualStreams, RMSNorm)
 from .decoder import LayerCall, ModelSpec
 
 SWISH_ALPHA = 1.702     # an expert's gate is g * sigmoid(SWISH_ALPHA * g)
@@ -58,14 +59,17 @@ def build_renapel(config: RenapelConfig) -> ModelSpec:
     for index, layer in enumerate(c.layers):
         p = f"l{index}."
         feed_forward = _feed_forward(layer["mlp"], p + "mlp.", c)
-        layers.append(HyperConnectionBlock(
-            c.streams, c.width, RMSNorm(p, c.width, c.norm_eps, name=p + "norm1"), _mixer(layer["type"], layer["mixer"], p + "mix.", c), p + "hc1.",
-            None if feed_forward is None else RMSNorm(p, c.width, c.norm_eps, name=p + "norm2"), feed_forward,
-            None if feed_forward is None else p + "hc2."))
+        norm1, mixer = RMSNorm(p, c.width, c.norm_eps, name=p + "norm1"), _mixer(layer["type"], layer["mixer"], p + "mix.", c)
+        norm2 = None if feed_forward is None else RMSNorm(p, c.width, c.norm_eps, name=p + "norm2")
+        if c.streams is None:
+            layers.append(PreNormBlock(norm1, mixer, norm2, feed_forward, unread=[] if feed_forward is not None else [p + "norm2"]))
+        else:
+            layers.append(HyperConnectionBlock(c.streams, c.width, norm1, mixer, p + "hc1.", norm2, feed_forward, p + "hc2.",
+                                               unread=[p + "norm2"]))
         schedule.append(LayerCall(index, reads_cache_of=layer["mixer"].get("kv_from") if layer["type"] == "attention" else None))
     return ModelSpec(config=c, embedding=Embedding("", c.vocab, c.width, name="embed"), layers=layers, schedule=schedule,
                      final_norm=RMSNorm("", c.width, c.norm_eps, name="final.norm"), head=OutputHead("", c.vocab, c.width, name="head"),
-                     streams=ResidualStreams(c.streams, c.width))
+                     streams=None if c.streams is None else ResidualStreams(c.streams, c.width))
 
 
 register_architecture("Renapel", RenapelConfig, build_renapel)

@@ -18,9 +18,10 @@ from .base import Block, CacheNeeds, Part, Runtime, WeightSpec, register_part
 
 
 class PreNormBlock(Block):
-    def __init__(self, mixer_norm, mixer, feed_forward_norm=None, feed_forward=None, mixer_input=None, feed_forward_input=None):
+    def __init__(self, mixer_norm, mixer, feed_forward_norm=None, feed_forward=None, mixer_input=None, feed_forward_input=None, unread=()):
         if (feed_forward is None) != (feed_forward_norm is None):
             raise ValueError("a feed-forward and its norm come together")
+        self.unread = list(unread)          # tensors that a checkpoint may carry for this block and that it does not read
         self.mixer_norm = mixer_norm
         self.mixer = mixer
         self.feed_forward_norm = feed_forward_norm
@@ -41,6 +42,9 @@ class PreNormBlock(Block):
         for part in self.parts():
             specs.update(part.weight_specs())
         return specs
+
+    def ignored_names(self):
+        return self.unread + [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
 
     def cache_needs(self) -> CacheNeeds:
         return self.mixer.cache_needs().merged(*[part.cache_needs() for part in (self.mixer_input, self.feed_forward_input)
@@ -270,7 +274,7 @@ class HyperConnectionBlock(Block):
     passes_norms = True
 
     def __init__(self, count: int, hidden: int, mixer_norm, mixer, mixer_connection: str, feed_forward_norm=None, feed_forward=None,
-                 feed_forward_connection: Optional[str] = None):
+                 feed_forward_connection: Optional[str] = None, unread=()):
         if (feed_forward is None) != (feed_forward_norm is None):
             raise ValueError("a feed-forward and its norm come together")
         if feed_forward is not None and feed_forward_connection is None:
@@ -279,6 +283,9 @@ class HyperConnectionBlock(Block):
         self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward = mixer_norm, mixer, feed_forward_norm, feed_forward
         self.connections = [mixer_connection] + ([feed_forward_connection] if feed_forward is not None else [])
         self.weights = []
+        # what a checkpoint may carry for a block without a feed-forward and nobody reads: the second connection's tensors, and `unread`
+        self.unread = [] if feed_forward is not None else (list(unread) + ([feed_forward_connection + name for name in ("in", "out", "mix")]
+                                                                          if feed_forward_connection is not None else []))
 
     def parts(self):
         return tuple(part for part in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward) if part is not None)
@@ -298,7 +305,7 @@ class HyperConnectionBlock(Block):
         return specs
 
     def ignored_names(self):
-        return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
+        return self.unread + [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
 
     def cache_needs(self) -> CacheNeeds:
         return self.mixer.cache_needs()
