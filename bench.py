@@ -37,6 +37,13 @@ the same for the Depunex decoder (layers of a matrix state per head with step si
 positions beside a selective scan, in turn; a clamped gated feed-forward or eight experts of which a token uses two, in
 turn; the hashed table of token pairs, the per-layer side input and the capped logits), beside the Sozopel decoder, the
 library's closest (recurrences, short convolutions, two mixers side by side on the general attention kernel), and Llama.
+
+    python bench.py --design renapel [--size small|medium|large] [--layers N]
+
+the same for the Renapel decoder (a residual stream in four copies; layers of lightning attention, of attention through a
+cached latent, and of softmax attention with a learnt sink and biases by distance, of which every second reads the keys and
+values of the one before it; eight clamped experts of which a token uses two after every mixer), beside the Depunex decoder,
+the library's closest (a matrix state per head, attention on the general kernel, experts), and Llama.
 """
 import argparse
 import json
@@ -165,8 +172,29 @@ def depunex_config(size, layers, max_positions):
             "layers": [kinds[i % 4] for i in range(layers)]}
 
 
-DESIGN_CONFIGS = {"sozopel": sozopel_config, "ledudra": ledudra_config, "depunex": depunex_config}
-DESIGN_BESIDE = {"depunex": ("sozopel", "llama")}          # the models a design is measured beside (Llama alone unless named)
+def renapel_config(size, layers, max_positions):
+    w, d, ff = size["width"], size["head"], size["ff"]
+    heads = w // d
+    experts = {"kind": "moe", "expert": {"ff": ff // 2, "limit": 7.0},
+               "router": {"experts": 8, "top": 2, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    lightning = {"heads": heads, "dim": d, "vdim": d, "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(heads)]}
+    attention = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": d, "vdim": d, "scale": d ** -0.5, "bias_max": 2048, "bias_rows": 32,
+                 "q_temp": {"coef": 0.1, "every": 1024}}
+    latent = {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "kv_rank": 3 * d, "q_rank": 6 * d, "scale": (3 * d // 2) ** -0.5,
+              "rot": {"dims": d // 2, "base": 500000.0}}
+    kinds = [("lightning", lightning), ("latent_attention", latent), ("attention", attention), ("lightning", lightning),
+             ("attention", None), ("latent_attention", latent)]
+    out = []
+    for i in range(layers):
+        kind, mixer = kinds[i % 6]
+        if mixer is None:                                   # the second attention layer of six reads the first one's keys and values
+            mixer = dict(attention, kv_from=i - 2)
+        out.append({"type": kind, "mixer": mixer, "mlp": experts})
+    return {"architecture": "Renapel", "vocab": size["vocab"], "width": w, "norm": {"eps": 1e-6}, "streams": 4, "layers": out}
+
+
+DESIGN_CONFIGS = {"sozopel": sozopel_config, "ledudra": ledudra_config, "depunex": depunex_config, "renapel": renapel_config}
+DESIGN_BESIDE = {"depunex": ("sozopel", "llama"), "renapel": ("depunex", "llama")}          # the models a design is measured beside (Llama alone unless named)
 
 
 def llama_config(size, layers, max_positions):
@@ -183,7 +211,7 @@ def run_design(args) -> int:
     layers = args.layers if args.layers is not None else 6
     context = DESIGN_CONTEXT
     most = max(DESIGN_BATCHES)
-    beside = DESIGN_BESIDE.get(args.design, ("llama",))
+    beside = () if args.alone else DESIGN_BESIDE.get(args.design, ("llama",))
     record = {"design": args.design, "beside": ", ".join(beside), "size": args.size, **size, "layers": layers, "dtype": args.dtype,
               "context": context, "prefill_tokens": PREFILL_TOKENS, "data": "synthetic token ids, random weights N(0, 0.02)"}
     configs = {**DESIGN_CONFIGS, "llama": llama_config}
@@ -357,6 +385,7 @@ def main() -> int:
     parser.add_argument("--design", default=None, choices=sorted(DESIGN_CONFIGS),
                         help="measure this design beside the Llama decoder of equal sizes instead (see the top of this file)")
     parser.add_argument("--size", default="medium", choices=sorted(DESIGN_SIZES), help="with --design: the layers' sizes")
+    parser.add_argument("--alone", action="store_true", help="with --design: the design's model only, not those beside it (for a profile)")
     parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                         help="with --phase prefill: the prompt's length (the record's prefill is always of 2048 tokens)")
     args = parser.parse_args()

@@ -202,6 +202,7 @@ class Step:
         self.positions = ints([start + t for start, count in zip(starts, counts) for t in range(count)])
         self.slots = ints([slot for slot, count in zip(slots, counts) for _ in range(count)])
         self.max_context = max(start + count for start, count in zip(starts, counts))
+        self.host_slots, self.host_counts, self.host_starts = list(slots), list(counts), list(starts)
 
 
 def schedules(length):
@@ -397,7 +398,10 @@ def test_attention_with_a_learnt_sink_and_a_bias_by_distance(n_heads, n_kv_heads
         got = attend(ops, q, k, v, cuts, dtype, n_heads, n_kv_heads, dim, vdim, scale=scale, sink=sink.cuda(), distance_bias=table.cuda())
         assert float((got - want).abs().max()) <= (1e-5 if dtype == torch.float32 else 2e-2) * float(want.abs().max()), f"cuts {cuts[:4]}"
         first = got if first is None else first
-        assert torch.equal(got, first), f"cuts {cuts[:4]} change the bits"
+        # (bfloat16 heads of 64 or 128 dims: steps of several tokens go to the matrix cores, steps of one token do not, and the
+        # two agree but for rounding)
+        if not (dtype == torch.bfloat16 and dim == vdim and dim in (64, 128)):
+            assert torch.equal(got, first), f"cuts {cuts[:4]} change the bits"
 
 
 def test_the_sink_takes_its_share_and_nothing_else(ops):
@@ -510,6 +514,23 @@ def test_latent_attention_alone(m, dtype, ops):
         got = run_mixer(part, h, cuts, cache, dtype)
         assert float((got - want).abs().max()) <= limit * float(want.abs().max()), f"cuts {cuts[:3]}"
     assert cache.kv.k.shape[1] == 1 and cache.kv.k.shape[3] == m["kv_rank"] + m["rot_dim"] and cache.kv.v.shape[2] == m["kv_rank"]
+    # prompts that start their sequences, nothing else in the step: in bfloat16 their scores are a matrix product of the step's own rows
+    if dtype == torch.bfloat16:
+        part.DENSE_SCORES = 70 * m["heads"] * length                 # (the prompt's queries in three stretches)
+    cache = layer_cache(part.cache_needs(), dtype, length)
+    assert part._prompts_alone(h.cuda(), Step([1], [length], [0]), cache) == (dtype == torch.bfloat16)
+    for cuts in ([length], [length - 20] + [1] * 20):
+        cache = layer_cache(part.cache_needs(), dtype, length)
+        got = run_mixer(part, h, cuts, cache, dtype, padding=0)
+        assert float((got - want).abs().max()) <= limit * float(want.abs().max()), f"prompts alone, cuts {cuts[:3]}"
+    # two prompts of unequal length in one step, against each alone
+    if dtype == torch.bfloat16:
+        cache = layer_cache(part.cache_needs(), dtype, length + 128)
+        cache.kv.block_table[0, :2] = torch.tensor([0, 1], dtype=torch.int32)      # (two blocks that the sequence in slot 1 does not reach)
+        both = torch.full((length + 70, part.hidden), float("nan"), device="cuda")
+        part.forward_into(torch.cat([h[:70], h]).to(dtype).cuda(), Step([0, 1], [70, length], [0, 0]), cache, both)
+        assert float((both[70:].double().cpu() - want).abs().max()) <= limit * float(want.abs().max())
+        assert float((both[:70].double().cpu() - want[:70]).abs().max()) <= limit * float(want.abs().max())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -575,6 +596,41 @@ def test_clamped_experts_alone(mlp, dtype, ops):
     alone = torch.empty(1, width, device="cuda")
     part.forward_into(h[17:18].cuda(), None, alone)
     assert float((alone[0] - out[17]).abs().max()) <= 1e-5 * float(want.abs().max()) if dtype == torch.float32 else True
+
+
+@pytest.mark.parametrize("ff,experts,top,groups,tokens", [(64, 8, 2, (4, 2), 300), (128, 16, 4, None, 1000), (192, 4, 1, (2, 1), 600)])
+def test_clamped_experts_multiply_only_the_tokens_that_chose_them(ff, experts, top, groups, tokens, ops):
+    """A step of many tokens sorts its picks by expert: against the plain sum, and against the same part with every token
+    through every expert (the same choices, so rounding alone differs)."""
+    from renapel_models import _moe
+    from xeno_rt_amd.models.renapel import _feed_forward
+    width = 64
+    raw = _moe(ff, 1.5, experts, top, groups, 2.0)
+    part = _feed_forward(raw, "mlp.", types.SimpleNamespace(width=width))
+    tensors = tensors_for(part, seed=ff, std=0.3, router=(0.0, 0.7))
+    part.bind(tensors, runtime(ops, torch.bfloat16))
+    h = torch.randn(tokens, width, generator=torch.Generator().manual_seed(6)).bfloat16()
+    assert ops.experts_sorted_takes(h.cuda(), part.w_gate_up, part.w_down, experts, ff, top, stacked=True)
+    assert not ops.experts_sorted_takes(h[:8].cuda(), part.w_gate_up, part.w_down, experts, ff, top, stacked=True)
+    out = torch.full((tokens, width), float("nan"), device="cuda")
+    part.forward_into(h.cuda(), None, out)
+    takes = ops.experts_sorted_takes
+    ops.experts_sorted_takes = lambda *operands, **options: False
+    try:
+        dense = torch.empty(tokens, width, device="cuda")
+        part.forward_into(h.cuda(), None, dense)
+    finally:
+        ops.experts_sorted_takes = takes
+    want = P.experts_ff(h.double(), short(tensors, "mlp."), raw)
+    scale = float(want.abs().max())
+    assert float((out - dense).abs().max()) <= 1e-2 * scale
+    per_row = (out.double().cpu() - want).abs().max(dim=1).values / scale
+    assert int((per_row > 3e-2).sum()) <= max(2, tokens // 50), f"rows {(per_row > 3e-2).nonzero().flatten().tolist()} differ from the plain sum"
+    some = torch.arange(tokens - 1, -1, -3)
+    fewer = torch.empty(len(some), width, device="cuda")
+    part.forward_into(h[some].cuda(), None, fewer)
+    if ops.experts_sorted_takes(h[some].cuda(), part.w_gate_up, part.w_down, experts, ff, top, stacked=True):
+        assert torch.equal(fewer, out[some.cuda()]), "a token's bits depend on its company"
 
 
 # ---- through the programs a user runs ----------------------------------------------------------------------------------

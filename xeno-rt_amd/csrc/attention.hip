@@ -20,7 +20,7 @@ bool xrt_attention_prefill_accepts(int head_dim);
 int xrt_attention_prefill(const void* qkv, long q_stride, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                           const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
-                          float scale, int stretch, bool fine, hipStream_t s);
+                          float scale, int stretch, bool fine, const float* bias, int span, const float* sinks, hipStream_t s);
 
 static bool takes_decode_kernel(int dtype, int n_heads, int n_kv_heads, int head_dim, int window, int max_count, int max_context) {
     return dtype == XRT_BF16 && window == 0 && max_count == 1 && max_context > 0 && n_heads > 0 && n_kv_heads > 0 &&
@@ -62,7 +62,7 @@ extern "C" int xrt_attention(const void* qkv, int dtype, int tokens, int n_heads
             XRT_REQUIRE(n_seqs <= tokens, "attention: more sequences than tokens");
             return xrt_attention_prefill(qkv, 0, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table,
                                          table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, out,
-                                         scale, 0, false, s);
+                                         scale, 0, false, nullptr, 0, nullptr, s);
         }
     }
     return xrt_attention_generic(qkv, dtype, tokens, n_heads, n_kv_heads, head_dim, head_dim, k_cache, v_cache, block_table,
@@ -105,7 +105,8 @@ extern "C" int xrt_attention_stretches_accepts(int dtype, int head_dim, int valu
 extern "C" int xrt_attention_stretches(const void* q, long q_stride, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                                        const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                                        const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
-                                       float scale, int chunk, void* stream) {
+                                       float scale, int chunk, const float* distance_bias, int bias_span, const float* sink_scores,
+                                       void* stream) {
     XRT_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention: head counts %d/%d: the first must be a multiple of the second", n_heads, n_kv_heads);
     XRT_REQUIRE(xrt_attention_stretches_accepts(dtype, head_dim, head_dim, chunk),
@@ -114,7 +115,8 @@ extern "C" int xrt_attention_stretches(const void* q, long q_stride, int dtype, 
     XRT_REQUIRE(table_stride > 0 && n_blocks > 0 && n_seqs > 0 && n_seqs <= tokens, "attention: empty cache, or no sequences");
     if (tokens == 0) return 0;
     return xrt_attention_prefill(q, q_stride, tokens, n_heads, n_kv_heads, head_dim, k_cache, v_cache, block_table, table_stride, n_blocks,
-                                 seq_offsets, seq_slots, seq_starts, n_seqs, out, scale, chunk, true, (hipStream_t)stream);
+                                 seq_offsets, seq_slots, seq_starts, n_seqs, out, scale, chunk, true, distance_bias, bias_span, sink_scores,
+                                 (hipStream_t)stream);
 }
 
 // ---- a decode step whose attention also finishes q, k and v (xrt_hip.h)

@@ -320,7 +320,9 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
     // few (token, head) pairs (a decode step): a workgroup of wavefronts each, which take the chunks of keys side by side
     const bool side_by_side = (long)tokens * n_heads <= 8L * XRT_COMPUTE_UNITS;
     const int sees_at_most = window > 0 && stretch > 0 ? min(window, stretch) : max(window, stretch);     // (0: everything)
-    const int chunk_blocks = sees_at_most > 0 && sees_at_most <= WINDOW_FOR_SHORT_CHUNKS ? 1 : CHUNK_BLOCKS;
+    // (bfloat16 also without a window: what its chunks cost in merges is little beside a decode step's wavefronts that would
+    // otherwise stand idle; the rule knows the element type and the window alone, which an engine fixes)
+    const int chunk_blocks = dtype == XRT_BF16 || (sees_at_most > 0 && sees_at_most <= WINDOW_FOR_SHORT_CHUNKS) ? 1 : CHUNK_BLOCKS;
     const size_t round_bytes = (size_t)2 * CHUNK_WAVES * together * value_dim * sizeof(float);
 #define XRT_GENERIC(T, WAVES_, G_, OWNED_)                                                                                \
     attention_generic_kernel<T, WAVES_, G_, OWNED_><<<(unsigned)items, WAVES_ * XRT_WAVE, WAVES_ > 1 ? round_bytes : 0, s>>>( \

@@ -52,12 +52,18 @@ constexpr int QW = GROUPS * QT;        // queries of a tile
 
 // FINE: the probabilities enter the value product as two bfloat16 numbers each, the rounded one and what the rounding left
 // (sixteen bits of them instead of eight, for twice the value products), for models whose weights are float32.
-template <int HD, bool FINE>
+// EXTRAS: a bias by distance (bias [n_heads][span] float32, or null: a key d tokens behind the query adds
+// bias[head][min(d, span - 1)] to its scaled score) and a sink (sinks [n_heads], or null: the softmax's denominator also holds
+// exp(sinks[head]), neither scaled nor biased); instantiated apart, so that the kernels without them stay as they are.
+struct PrefillExtras {
+    const float* bias; int span; float inv_scale; const float* sinks;
+};
+template <int HD, bool FINE, bool EXTRAS = false>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     const bf16* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads,
     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ seq_offsets, const int* __restrict__ seq_slots,
-    const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale, int stretch) {
+    const int* __restrict__ seq_starts, int n_seqs, bf16* __restrict__ out, float scale, int stretch, const PrefillExtras extras) {
     constexpr int KS = HD / 16;            // K steps of the score product
     constexpr int DT = HD / 32;            // 32-row tiles of the value product
     constexpr int K_CHUNKS = HD / 8;       // 16-byte chunks of a key row (16 or 8)
@@ -149,6 +155,9 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
     // the result of the queries at hand: out = o / l
     auto write_out = [&]() {
         if (!q_valid) return;
+        if constexpr (EXTRAS) {                              // the sink joins the sum, relative to the same exponent as the keys' terms
+            if (extras.sinks != nullptr) l += __builtin_amdgcn_exp2f(fmaf(extras.sinks[head], LOG2E, -(m == -INFINITY ? 0.f : m)));
+        }
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         bf16* dst = out + (token * n_heads + head) * HD;
         // accumulator register i of tile dt is dimension dt*32 + (i/4)*8 + half*4 + i%4, for this lane's query
@@ -255,6 +264,16 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         fetch_piece();
 
         // register i is key k0 + (i/8)*16 + half*8 + i%8, for this lane's query
+        if constexpr (EXTRAS) {
+            if (extras.bias != nullptr) {                    // (in units of the raw products: the scale multiplies them later)
+                const float* of_head = extras.bias + (long)head * extras.span;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int behind = q_pos - (k0 + (i / 8) * 16 + half * 8 + i % 8);
+                    s[i] = fmaf(of_head[min(max(behind, 0), extras.span - 1)], extras.inv_scale, s[i]);
+                }
+            }
+        }
         if (edge) {
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -383,15 +402,16 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_prefill_kernel(
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) o[dt][e] = o[dt][e] * mine + merge_o[group][dt * 16 + e][lane] * theirs;
+        m = m_all;                                           // what l and o are relative to now
     }
     l += __shfl_xor(l, 32, XRT_WAVE);
     write_out();
 }
 
-template <int HD, bool FINE>
+template <int HD, bool FINE, bool EXTRAS = false>
 int launch_waves(const bf16* qkv, long q_stride, int tokens, int n_heads, int n_kv_heads, const bf16* k_cache, const bf16* v_cache,
                  const int* block_table, int table_stride, int n_blocks, const int* seq_offsets, const int* seq_slots,
-                 const int* seq_starts, int n_seqs, bf16* out, float scale, int stretch, hipStream_t s) {
+                 const int* seq_starts, int n_seqs, bf16* out, float scale, int stretch, const PrefillExtras& extras, hipStream_t s) {
     const int row_width = q_stride > 0 ? (int)q_stride : (n_heads + 2 * n_kv_heads) * HD;
     // a run of `count` tokens has ceil(ceil(count / QW) / 2) pairs of tiles; their sum is at most this. A sequence is one run,
     // or with stretches of positions a run per stretch that its new tokens touch.
@@ -403,14 +423,14 @@ int launch_waves(const bf16* qkv, long q_stride, int tokens, int n_heads, int n_
     static_assert(lds >= GROUPS * (HD / 32 * 16 + 2) * XRT_WAVE * sizeof(float), "the merge does not fit the blocks' buffers");
     static bool configured = false;          // per instantiation
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD, FINE>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_prefill_kernel<HD, FINE, EXTRAS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         XRT_REQUIRE(e == hipSuccess, "attention (prefill): cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         configured = true;
     }
-    attention_prefill_kernel<HD, FINE><<<grid, WAVES * XRT_WAVE, lds, s>>>(
+    attention_prefill_kernel<HD, FINE, EXTRAS><<<grid, WAVES * XRT_WAVE, lds, s>>>(
         qkv, row_width, n_heads, n_kv_heads, k_cache, v_cache, block_table, table_stride, n_blocks, seq_offsets,
-        seq_slots, seq_starts, n_seqs, out, scale, stretch);
+        seq_slots, seq_starts, n_seqs, out, scale, stretch, extras);
     XRT_LAUNCH_CHECK("attention (prefill)");
     return 0;
 }
@@ -421,17 +441,24 @@ bool xrt_attention_prefill_accepts(int head_dim) { return head_dim == 64 || head
 
 // q_stride: 0, or how far the rows of q lie apart when they hold the queries alone. stretch: 0, or the size of the stretches
 // that positions are cut into (a multiple of the cache block), of which a query sees its own. fine: probabilities of sixteen bits.
+// bias (float32 [n_heads][span], or null) and sinks (float32 [n_heads], or null): see PrefillExtras.
 int xrt_attention_prefill(const void* qkv, long q_stride, int tokens, int n_heads, int n_kv_heads, int head_dim, const void* k_cache,
                           const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
-                          float scale, int stretch, bool fine, hipStream_t s) {
+                          float scale, int stretch, bool fine, const float* bias, int span, const float* sinks, hipStream_t s) {
+    XRT_REQUIRE((bias == nullptr || span > 0) && scale > 0.f, "attention (prefill): a table of biases needs a distance at least, and the scale is positive");
+    const PrefillExtras extras{bias, span, 1.0f / scale, sinks};
     XRT_REQUIRE(stretch >= 0 && stretch % BT == 0, "attention (prefill): stretches of %d positions are not whole cache blocks", stretch);
     XRT_REQUIRE(q_stride == 0 || (q_stride >= (long)n_heads * head_dim && q_stride % 8 == 0 && q_stride <= INT_MAX),
                 "attention (prefill): rows of q %ld apart", q_stride);
     auto run = [&](auto launcher) {
         return launcher((const bf16*)qkv, q_stride, tokens, n_heads, n_kv_heads, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
-                        table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, stretch, s);
+                        table_stride, n_blocks, seq_offsets, seq_slots, seq_starts, n_seqs, (bf16*)out, scale, stretch, extras, s);
     };
+    if (bias != nullptr || sinks != nullptr) {               // (served with probabilities of sixteen bits)
+        XRT_REQUIRE(fine, "attention (prefill): biases by distance and sinks go with probabilities of sixteen bits");
+        return head_dim == 64 ? run(launch_waves<64, true, true>) : run(launch_waves<128, true, true>);
+    }
     if (head_dim == 64) return fine ? run(launch_waves<64, true>) : run(launch_waves<64, false>);
     return fine ? run(launch_waves<128, true>) : run(launch_waves<128, false>);
 }

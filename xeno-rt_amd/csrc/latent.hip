@@ -9,6 +9,12 @@
 //   xrt_latent_queries   from the queries' float32 sums, head by head [plain | part to turn]: the plain parts to rows of
 //                        their own, the turned parts to the tail of the rows that the attention kernel reads
 //   xrt_linear_heads     out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k], float32 sums in the order of k
+// A prompt that starts a sequence can have its scores as a matrix product of its own rows (all heads' queries of a stretch of
+// tokens against the prompt's cached rows, which the step has at hand): then
+//   xrt_causal_softmax   turns the float32 scores [queries x heads][keys] into the softmax's weights over the keys at or before
+//                        each query, with the heads' sinks in the denominators, as two bfloat16 numbers each (the rounded weight
+//                        and what the rounding left) for the product with the latents
+//   xrt_transpose        dst[c][r] = src[r][c]: the latents with the tokens along the rows, as that product wants them
 #include "cache_layout.h"
 #include "xrt_hip.h"
 
@@ -32,11 +38,15 @@ __global__ void __launch_bounds__(256) latent_complete_kernel(const float* __res
                                                              const void* __restrict__ gain, int gain_dtype, float eps,
                                                              const float* __restrict__ frequencies, const int* __restrict__ positions,
                                                              const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                                             const int* __restrict__ block_table, int table_stride, int n_blocks) {
+                                                             const int* __restrict__ block_table, int table_stride, int n_blocks,
+                                                             T* __restrict__ rows_out) {
     __shared__ float scratch[32];
     const long t = blockIdx.x;
     const int slot = slots[t], pos = positions[t];
-    if (slot < 0) return;                                      // (the whole workgroup)
+    if (slot < 0) {                                            // (the whole workgroup)
+        if (rows_out != nullptr) for (int e = threadIdx.x; e < rank + rot_dim; e += blockDim.x) rows_out[t * (rank + rot_dim) + e] = from_float<T>(0.f);
+        return;
+    }
     const int block = block_table[(long)slot * table_stride + pos / XRT_BLOCK_TOKENS];
     if (block < 0 || block >= n_blocks) return;
     const float* row = down + t * down_stride;
@@ -51,8 +61,11 @@ __global__ void __launch_bounds__(256) latent_complete_kernel(const float* __res
             const T c = from_float<T>(row[e] * inv * small_at(gain, gain_dtype, e));
             keys[cache_key_offset(place, e, head_dim)] = c;
             values[cache_value_offset(e, place, rank)] = c;
+            if (rows_out != nullptr) rows_out[t * head_dim + e] = c;
         } else {
-            keys[cache_key_offset(place, e, head_dim)] = from_float<T>(turned(row + rank, e - rank, rot_dims, frequencies, pos));
+            const T k = from_float<T>(turned(row + rank, e - rank, rot_dims, frequencies, pos));
+            keys[cache_key_offset(place, e, head_dim)] = k;
+            if (rows_out != nullptr) rows_out[t * head_dim + e] = k;
         }
     }
 }
@@ -118,11 +131,117 @@ __global__ void __launch_bounds__(256) linear_heads_kernel(const T* __restrict__
         }
 }
 
+// A workgroup a row: row m is the query at position first_position + m / heads of head m % heads. Three passes over the row
+// (largest visible score, sum, weights); keys behind the query's position get a weight of nothing.
+__global__ void __launch_bounds__(256) causal_softmax_kernel(const float* __restrict__ scores, long keys, int heads, int first_position, float scale,
+                                                            const float* __restrict__ sinks, bf16* __restrict__ rounded, bf16* __restrict__ rest) {
+    __shared__ float scratch[32];
+    const long row = blockIdx.x;
+    const int head = (int)(row % heads), visible = min((long)first_position + row / heads + 1, keys);
+    const float* mine = scores + row * keys;
+    const float sink = sinks != nullptr ? sinks[head] : -INFINITY;
+    float top = sink;
+    for (int j = threadIdx.x; j < visible; j += 256) top = fmaxf(top, mine[j] * scale);
+    top = wave_max(top);
+    __syncthreads();
+    if (threadIdx.x % XRT_WAVE == 0) scratch[threadIdx.x / XRT_WAVE] = top;
+    __syncthreads();
+    for (int w = 0; w < 256 / XRT_WAVE; ++w) top = fmaxf(top, scratch[w]);
+    float sum = 0.f;
+    for (int j = threadIdx.x; j < visible; j += 256) sum += expf(mine[j] * scale - top);
+    sum = block_sum(sum, scratch);
+    if (sinks != nullptr) sum += expf(sink - top);
+    const float inv = 1.0f / sum;
+    for (long j = threadIdx.x; j < keys; j += 256) {
+        const float weight = j < visible ? expf(mine[j] * scale - top) * inv : 0.f;
+        const bf16 first = from_float<bf16>(weight);
+        rounded[row * keys + j] = first;
+        rest[row * keys + j] = from_float<bf16>(weight - to_float(first));
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ src, long src_stride, long rows, int cols, T* __restrict__ dst) {
+    __shared__ T tile[32][33];
+    const long r0 = (long)blockIdx.x * 32;
+    const int c0 = blockIdx.y * 32, tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+    for (int i = ty; i < 32; i += 8)
+        if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = src[(r0 + i) * src_stride + c0 + tx];
+    __syncthreads();
+    for (int i = ty; i < 32; i += 8)
+        if (c0 + i < cols && r0 + tx < rows) dst[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
+}
+
+// The same product for a step of few rows (a decode step): a lane an output, the rows of a in LDS, the lane's row of w read
+// sixteen bytes at a time; every output's sum runs over k in the same order as in the tiles above, to the same bits.
+constexpr int HEADS_FEW = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(XRT_WAVE) linear_heads_few_kernel(const T* __restrict__ a, long a_stride, long a_head, const T* __restrict__ w,
+                                                                   T* __restrict__ out, long out_stride, long out_head, int rows, int n, int k) {
+    extern __shared__ float rows_of_a[];                       // [rows][k]
+    const int head = blockIdx.y, lane = threadIdx.x, column = blockIdx.x * XRT_WAVE + lane;
+    for (int e = lane; e < rows * k; e += XRT_WAVE) rows_of_a[e] = to_float(a[(long)(e / k) * a_stride + (long)head * a_head + e % k]);
+    wave_sync();
+    if (column >= n) return;
+    const T* mine = w + ((long)head * n + column) * k;
+    float acc[HEADS_FEW];
+#pragma unroll
+    for (int r = 0; r < HEADS_FEW; ++r) acc[r] = 0.f;
+    constexpr int PIECE = 16 / sizeof(T);
+    const bool whole = k % PIECE == 0 && (uintptr_t)w % 16 == 0;
+    for (int k0 = 0; k0 < k; k0 += PIECE) {
+        float piece[PIECE];
+        if (whole) {
+            struct alignas(16) Piece { T e[PIECE]; };
+            const Piece loaded = *reinterpret_cast<const Piece*>(mine + k0);
+#pragma unroll
+            for (int e = 0; e < PIECE; ++e) piece[e] = to_float(loaded.e[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < PIECE; ++e) piece[e] = k0 + e < k ? to_float(mine[k0 + e]) : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < PIECE; ++e) {
+            if (k0 + e < k) {
+#pragma unroll
+                for (int r = 0; r < HEADS_FEW; ++r)
+                    if (r < rows) acc[r] = fmaf(rows_of_a[r * k + k0 + e], piece[e], acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < HEADS_FEW; ++r)
+        if (r < rows) out[(long)r * out_stride + (long)head * out_head + column] = from_float<T>(acc[r]);
+}
+
 }  // namespace
+
+extern "C" int xrt_causal_softmax(const float* scores, long rows, long keys, int heads, int first_position, float scale, const float* sinks,
+                                  void* rounded, void* rest, void* stream) {
+    XRT_REQUIRE(scores && rounded && rest && rows >= 0 && rows < (1L << 31) && keys > 0 && keys < (1L << 31) && heads > 0 && first_position >= 0,
+                "causal_softmax: bad operands");
+    if (rows == 0) return 0;
+    causal_softmax_kernel<<<(unsigned)rows, 256, 0, (hipStream_t)stream>>>(scores, keys, heads, first_position, scale, sinks, (bf16*)rounded, (bf16*)rest);
+    XRT_LAUNCH_CHECK("causal_softmax");
+    return 0;
+}
+
+extern "C" int xrt_transpose(const void* src, long src_stride, int dtype, long rows, int cols, void* dst, void* stream) {
+    XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "transpose: unknown dtype %d", dtype);
+    XRT_REQUIRE(src && dst && rows >= 0 && cols > 0 && src_stride >= cols && (rows + 31) / 32 < (1L << 31) && (cols + 31) / 32 <= 65535, "transpose: bad operands");
+    if (rows == 0) return 0;
+    const dim3 grid((unsigned)((rows + 31) / 32), (cols + 31) / 32);
+    if (dtype == XRT_F32) transpose_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)src, src_stride, rows, cols, (float*)dst);
+    else transpose_kernel<bf16><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16*)src, src_stride, rows, cols, (bf16*)dst);
+    XRT_LAUNCH_CHECK("transpose");
+    return 0;
+}
 
 extern "C" int xrt_latent_complete(const float* down, long down_stride, int dtype, long tokens, int rank, int rot_dim, int rot_dims,
                                    const void* gain, int gain_dtype, float eps, const float* frequencies, const int* positions, const int* slots,
-                                   void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks, void* stream) {
+                                   void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks, void* rows_out,
+                                   void* stream) {
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "latent_complete: unknown dtype %d", dtype);
     XRT_REQUIRE(gain_dtype == XRT_F32 || gain_dtype == XRT_BF16, "latent_complete: unknown dtype %d of the gain", gain_dtype);
     XRT_REQUIRE(down && gain && positions && slots && k_cache && v_cache && block_table, "latent_complete: null operand");
@@ -134,11 +253,11 @@ extern "C" int xrt_latent_complete(const float* down, long down_stride, int dtyp
     if (dtype == XRT_F32)
         latent_complete_kernel<float><<<(unsigned)tokens, 256, 0, (hipStream_t)stream>>>(down, down_stride, rank, rot_dim, rot_dims, gain, gain_dtype, eps,
                                                                                       frequencies, positions, slots, (float*)k_cache, (float*)v_cache,
-                                                                                      block_table, table_stride, n_blocks);
+                                                                                      block_table, table_stride, n_blocks, (float*)rows_out);
     else
         latent_complete_kernel<bf16><<<(unsigned)tokens, 256, 0, (hipStream_t)stream>>>(down, down_stride, rank, rot_dim, rot_dims, gain, gain_dtype, eps,
                                                                                      frequencies, positions, slots, (bf16*)k_cache, (bf16*)v_cache,
-                                                                                     block_table, table_stride, n_blocks);
+                                                                                     block_table, table_stride, n_blocks, (bf16*)rows_out);
     XRT_LAUNCH_CHECK("latent_complete");
     return 0;
 }
@@ -170,6 +289,18 @@ extern "C" int xrt_linear_heads(const void* a, long a_stride, long a_head, const
     XRT_REQUIRE(a_head >= k && a_stride >= (heads - 1) * a_head + k && out_head >= n && out_stride >= (heads - 1) * out_head + n,
                 "linear_heads: rows %ld and %ld apart do not hold %d heads %ld and %ld apart", a_stride, out_stride, heads, a_head, out_head);
     if (rows == 0) return 0;
+    if (rows <= HEADS_FEW && (size_t)rows * k * sizeof(float) <= 48 * 1024) {
+        const dim3 few((n + XRT_WAVE - 1) / XRT_WAVE, heads);
+        const size_t lds = (size_t)rows * k * sizeof(float);
+        if (dtype == XRT_F32)
+            linear_heads_few_kernel<float><<<few, XRT_WAVE, lds, (hipStream_t)stream>>>((const float*)a, a_stride, a_head, (const float*)w, (float*)out,
+                                                                                      out_stride, out_head, (int)rows, n, k);
+        else
+            linear_heads_few_kernel<bf16><<<few, XRT_WAVE, lds, (hipStream_t)stream>>>((const bf16*)a, a_stride, a_head, (const bf16*)w, (bf16*)out,
+                                                                                     out_stride, out_head, (int)rows, n, k);
+        XRT_LAUNCH_CHECK("linear_heads");
+        return 0;
+    }
     const long row_tiles = (rows + HEADS_TILE - 1) / HEADS_TILE;
     XRT_REQUIRE(row_tiles < (1L << 31) && (n + HEADS_TILE - 1) / HEADS_TILE <= 65535, "linear_heads: too many tiles");
     const dim3 grid((unsigned)row_tiles, (n + HEADS_TILE - 1) / HEADS_TILE, heads);

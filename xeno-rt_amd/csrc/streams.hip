@@ -11,7 +11,7 @@
 
 namespace {
 
-constexpr int STREAM_THREADS = 256;
+constexpr int STREAM_THREADS = 1024;         // the most threads of a workgroup; rows narrower than 2048 take 256
 constexpr int MOST_COPIES = XRT_MOST_STREAMS;
 
 __device__ __forceinline__ float gain_at(const void* p, int dtype, int i) {
@@ -23,7 +23,7 @@ __device__ __forceinline__ void store_as(void* p, int dtype, long i, float v) {
 
 __global__ void __launch_bounds__(STREAM_THREADS) streams_open_kernel(const float* __restrict__ x, float* __restrict__ streams, int width, int copies) {
     const long t = blockIdx.x;
-    for (int c = threadIdx.x; c < width; c += STREAM_THREADS) {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
         const float v = x[t * width + c];
         for (int s = 0; s < copies; ++s) streams[(t * copies + s) * width + c] = v;
     }
@@ -33,11 +33,11 @@ __global__ void __launch_bounds__(STREAM_THREADS) streams_open_kernel(const floa
 __device__ __forceinline__ void write_normed(const float* u, float squares, int width, const void* gain, int gain_dtype, float eps, void* out,
                                              int out_dtype, long to, float* scratch) {
     if (gain == nullptr) {
-        for (int c = threadIdx.x; c < width; c += STREAM_THREADS) store_as(out, out_dtype, to * width + c, u[c]);
+        for (int c = threadIdx.x; c < width; c += blockDim.x) store_as(out, out_dtype, to * width + c, u[c]);
         return;
     }
     const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)width + eps);
-    for (int c = threadIdx.x; c < width; c += STREAM_THREADS) store_as(out, out_dtype, to * width + c, u[c] * inv * gain_at(gain, gain_dtype, c));
+    for (int c = threadIdx.x; c < width; c += blockDim.x) store_as(out, out_dtype, to * width + c, u[c] * inv * gain_at(gain, gain_dtype, c));
 }
 
 __global__ void __launch_bounds__(STREAM_THREADS) streams_read_kernel(const float* __restrict__ streams, int copies, const float* __restrict__ in,
@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(STREAM_THREADS) streams_read_kernel(const floa
     __shared__ float scratch[32];
     const long t = rows != nullptr ? rows[blockIdx.x] : blockIdx.x;
     float squares = 0.f;
-    for (int c = threadIdx.x; c < width; c += STREAM_THREADS) {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
         float sum = 0.f;
         for (int s = 0; s < copies; ++s) sum = fmaf(in[s], streams[(t * copies + s) * width + c], sum);
         u[c] = sum;
@@ -66,12 +66,12 @@ __global__ void __launch_bounds__(STREAM_THREADS) streams_write_kernel(float* __
     float* mixes = weights;                                    // [from][to]
     float* outs = weights + MOST_COPIES * MOST_COPIES;
     float* ins = outs + MOST_COPIES;
-    for (int i = threadIdx.x; i < copies * copies; i += STREAM_THREADS) mixes[i] = mix[i];
-    for (int i = threadIdx.x; i < copies; i += STREAM_THREADS) { outs[i] = out_weights[i]; ins[i] = next_in != nullptr ? next_in[i] : 0.f; }
+    for (int i = threadIdx.x; i < copies * copies; i += blockDim.x) mixes[i] = mix[i];
+    for (int i = threadIdx.x; i < copies; i += blockDim.x) { outs[i] = out_weights[i]; ins[i] = next_in != nullptr ? next_in[i] : 0.f; }
     __syncthreads();
     const long t = blockIdx.x;
     float squares = 0.f;
-    for (int c = threadIdx.x; c < width; c += STREAM_THREADS) {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
         float old[MOST_COPIES];
 #pragma unroll
         for (int s = 0; s < MOST_COPIES; ++s) old[s] = s < copies ? streams[(t * copies + s) * width + c] : 0.f;
@@ -97,13 +97,15 @@ __global__ void __launch_bounds__(STREAM_THREADS) streams_write_kernel(float* __
     if (next_in != nullptr) write_normed(u, squares, width, gain, gain_dtype, eps, normed, normed_dtype, t, scratch);
 }
 
+int threads_for(int width) { return width >= 2048 ? STREAM_THREADS : 256; }
+
 }  // namespace
 
 extern "C" int xrt_streams_open(const float* x, float* streams, long tokens, int width, int copies, void* stream) {
     XRT_REQUIRE(x && streams && tokens >= 0 && tokens < (1L << 31) && width > 0 && copies > 0 && copies <= MOST_COPIES,
                 "streams_open: bad operands (%ld tokens, width %d, %d copies of up to %d)", tokens, width, copies, MOST_COPIES);
     if (tokens == 0) return 0;
-    streams_open_kernel<<<(unsigned)tokens, STREAM_THREADS, 0, (hipStream_t)stream>>>(x, streams, width, copies);
+    streams_open_kernel<<<(unsigned)tokens, threads_for(width), 0, (hipStream_t)stream>>>(x, streams, width, copies);
     XRT_LAUNCH_CHECK("streams_open");
     return 0;
 }
@@ -114,7 +116,7 @@ extern "C" int xrt_streams_read(const float* streams, int copies, const float* i
                 "streams_read: bad operands (%ld rows, width %d of up to 16384, %d copies of up to %d)", n_rows, width, copies, MOST_COPIES);
     XRT_REQUIRE((out_dtype == XRT_F32 || out_dtype == XRT_BF16) && (gain_dtype == XRT_F32 || gain_dtype == XRT_BF16), "streams_read: unknown dtype");
     if (n_rows == 0) return 0;
-    streams_read_kernel<<<(unsigned)n_rows, STREAM_THREADS, (size_t)width * sizeof(float), (hipStream_t)stream>>>(streams, copies, in, gain, gain_dtype,
+    streams_read_kernel<<<(unsigned)n_rows, threads_for(width), (size_t)width * sizeof(float), (hipStream_t)stream>>>(streams, copies, in, gain, gain_dtype,
                                                                                                                 eps, out, out_dtype, rows, width);
     XRT_LAUNCH_CHECK("streams_read");
     return 0;
@@ -129,7 +131,7 @@ extern "C" int xrt_streams_write(float* streams, int copies, const float* mix, c
     XRT_REQUIRE(next_in == nullptr || ((normed_dtype == XRT_F32 || normed_dtype == XRT_BF16) && (gain_dtype == XRT_F32 || gain_dtype == XRT_BF16)),
                 "streams_write: unknown dtype");
     if (tokens == 0) return 0;
-    streams_write_kernel<<<(unsigned)tokens, STREAM_THREADS, next_in != nullptr ? (size_t)width * sizeof(float) : 0, (hipStream_t)stream>>>(
+    streams_write_kernel<<<(unsigned)tokens, threads_for(width), next_in != nullptr ? (size_t)width * sizeof(float) : 0, (hipStream_t)stream>>>(
         streams, copies, mix, out_weights, y, width, next_in, gain, gain_dtype, eps, normed, normed_dtype);
     XRT_LAUNCH_CHECK("streams_write");
     return 0;

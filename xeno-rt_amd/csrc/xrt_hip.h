@@ -292,12 +292,13 @@ int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, i
 // The matrix-core attention for a step that brings sequences of many tokens, with the queries alone in q (rows q_stride
 // apart; keys and values are in the cache) and, with chunk > 0, queries that see the keys of their own stretch of `chunk`
 // positions only. `accepts` says which element type, head sizes and stretches it serves (stretches of whole cache blocks).
-// Tokens of the step that belong to no sequence keep what `out` held.
+// Tokens of the step that belong to no sequence keep what `out` held. distance_bias (float32 [n_heads][bias_span], or null) and
+// sink_scores (float32 [n_heads], or null) as in xrt_attention_general.
 int xrt_attention_stretches_accepts(int dtype, int head_dim, int value_dim, int chunk);
 int xrt_attention_stretches(const void* q, long q_stride, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
                             const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                             const int* seq_offsets, const int* seq_slots, const int* seq_starts, int n_seqs, void* out,
-                            float scale, int chunk, void* stream);
+                            float scale, int chunk, const float* distance_bias, int bias_span, const float* sink_scores, void* stream);
 
 // Attention without a softmax: the weight of a visible key is sigmoid(score_h + head_bias[h]), not normalised over the keys;
 // before that the heads' scaled scores of a (query, key) pair are mixed, score_h <- sum_g head_mix[h][g] score_g
@@ -441,14 +442,22 @@ int xrt_streams_write(float* streams, int copies, const float* mix, const float*
 // ---- attention through a latent (csrc/latent.hip) ---------------------------------------------------------------------------
 // The cache of such a layer has one key/value head whose keys are [latent (rank) | turned key part (rot_dim)] and whose values
 // are the latent. complete: from float32 rows [latent | key part] (down_stride apart) the latent / rms(latent) * gain and the
-// key part with its first rot_dims turned in pairs of neighbours by position * frequencies[pair], into the cache.
+// key part with its first rot_dims turned in pairs of neighbours by position * frequencies[pair], into the cache, and, with
+// rows_out, once more as rows [tokens][rank + rot_dim] of the cache's element type (zeros for tokens of no sequence).
 // queries: from float32 rows of heads x [plain (dim) | part to turn (rot_dim)] the plain parts to `plain` [tokens][heads][dim]
 // and the turned parts to full[t][h][rank ..], rows full_stride apart, heads rank + rot_dim apart.
 // linear_heads: out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k]; rows of a and out a_stride and out_stride apart, heads
 // a_head and out_head apart; all three of `dtype`, float32 sums in the order of k.
 int xrt_latent_complete(const float* down, long down_stride, int dtype, long tokens, int rank, int rot_dim, int rot_dims,
                         const void* gain, int gain_dtype, float eps, const float* frequencies, const int* positions, const int* slots,
-                        void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks, void* stream);
+                        void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks, void* rows_out, void* stream);
+// causal_softmax: scores float32 [rows][keys], row m being the query at position first_position + m / heads of head m % heads;
+// rounded and rest (bfloat16, same shape) get the weight of every key at or before the query, exp(score * scale) over the sum
+// of those and exp(sinks[head]) (sinks float32 [heads], or null), as the rounded number and what the rounding left; 0 elsewhere.
+// transpose: dst[c][r] = src[r][c] for r < rows, c < cols; rows of src src_stride apart, dst [cols][rows].
+int xrt_causal_softmax(const float* scores, long rows, long keys, int heads, int first_position, float scale, const float* sinks,
+                       void* rounded, void* rest, void* stream);
+int xrt_transpose(const void* src, long src_stride, int dtype, long rows, int cols, void* dst, void* stream);
 int xrt_latent_queries(const float* q, long q_stride, int dtype, long tokens, int heads, int dim, int rot_dim, int rot_dims,
                        const float* frequencies, const int* positions, void* plain, void* full, long full_stride, int rank, void* stream);
 int xrt_linear_heads(const void* a, long a_stride, long a_head, const void* w, int dtype, void* out, long out_stride, long out_head,

@@ -202,7 +202,7 @@ class HipOps:
                      "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts",
                      "xrt_experts_sort", "xrt_gather_rows", "xrt_linear_groups", "xrt_linear_groups_accepts", "xrt_experts_combine",
                      "xrt_linear_groups_tile_rows", "xrt_linear_groups_parts", "xrt_streams_open", "xrt_streams_read", "xrt_streams_write",
-                     "xrt_latent_complete", "xrt_latent_queries", "xrt_linear_heads"):
+                     "xrt_latent_complete", "xrt_latent_queries", "xrt_linear_heads", "xrt_causal_softmax", "xrt_transpose"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -500,8 +500,9 @@ class HipOps:
         from ..cache import BLOCK_TOKENS
         if finish is not None:
             return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
-        if (queries_alone and sink is False and distance_bias is None and distance_slopes is None and not window
-                and self._attention_stretches(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, chunk)):
+        if (queries_alone and sink is not True and distance_slopes is None and not window
+                and self._attention_stretches(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, chunk,
+                                              distance_bias, sink if isinstance(sink, torch.Tensor) else None)):
             return None
         if sink is not False or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone or chunk:
             return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
@@ -539,7 +540,8 @@ class HipOps:
             ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
-    def _attention_stretches(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, chunk) -> bool:
+    def _attention_stretches(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, chunk, distance_bias=None,
+                             sink_scores=None) -> bool:
         """The matrix-core kernel for a step that brings some sequence several tokens, the queries alone in `q`, every query
         seeing its own stretch of `chunk` positions (or, chunk None, all keys before it). False: not served here (another
         element type or head size, stretches that are not whole cache blocks, a step that is not described by sequences, or
@@ -566,10 +568,16 @@ class HipOps:
         counts = getattr(batch, "host_counts", None)
         if counts is None or sum(counts) < tokens:
             out.zero_()                       # padding rows: written by no one, read by the product that follows
+        span = 0
+        if distance_bias is not None:
+            span = distance_bias.shape[-1]
+            self._require(distance_bias, "attention distance_bias", torch.float32, (n_heads, span), q)
+        if sink_scores is not None:
+            self._require(sink_scores, "attention sink", torch.float32, (n_heads,), q)
         self._check(self.lib.xrt_attention_stretches(
             _ptr(q), ctypes.c_long(q_stride), _code(q), tokens, n_heads, n_kv_heads, head_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table),
             stride, n_blocks, _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs, _ptr(out), ctypes.c_float(scale), int(chunk or 0),
-            self._stream(q)))
+            _ptr(distance_bias), int(span), _ptr(sink_scores), self._stream(q)))
         return True
 
     def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink,
@@ -1047,13 +1055,15 @@ class HipOps:
                                                0 if out is None else _code(out), self._stream(streams)))
 
     # -- attention through a latent -----------------------------------------------------------------------
-    def latent_complete(self, down, rank, rot_dim, gain, eps, frequencies, rot_dims, kv, batch, like):
+    def latent_complete(self, down, rank, rot_dim, gain, eps, frequencies, rot_dims, kv, batch, like, rows_out=None):
         """From the float32 rows `down` [latent (rank) | key part (rot_dim)] (columns of a wider matrix will do): the latent divided
         by its root mean square, times gain, and the key part with its first rot_dims turned in pairs of neighbours by
         position * frequencies[pair], into the cache `kv` of one key/value head (keys rank + rot_dim wide, values rank wide), whose
-        element type is that of `like`."""
+        element type is that of `like`. rows_out ([tokens, rank + rot_dim] of that type, or None) takes the same rows once more."""
         tokens = down.shape[0]
         stride = self._rows(down, "latent_complete down", rank + rot_dim, torch.float32)
+        if rows_out is not None:
+            self._require(rows_out, "latent_complete rows_out", like.dtype, (tokens, rank + rot_dim), down)
         self._require(gain, "latent_complete gain", None, (rank,), down)
         if rot_dims:
             self._require(frequencies, "latent_complete frequencies", torch.float32, (rot_dims // 2,), down)
@@ -1063,7 +1073,28 @@ class HipOps:
         self._check(self.lib.xrt_latent_complete(_ptr(down), ctypes.c_long(stride), _code(like), ctypes.c_long(tokens), rank, rot_dim, int(rot_dims),
                                                  _ptr(gain), _code(gain), ctypes.c_float(eps), _ptr(frequencies), _ptr(batch.positions),
                                                  _ptr(batch.slots), _ptr(k_cache), _ptr(v_cache), _ptr(table), table_stride, n_blocks,
-                                                 self._stream(down)))
+                                                 _ptr(rows_out), self._stream(down)))
+
+    def causal_softmax(self, scores, heads, first_position, scale, sinks, rounded, rest):
+        """scores float32 [queries * heads, keys], row m the query at position first_position + m // heads of head m % heads:
+        the softmax's weights over the keys at or before the query (score * scale; sinks float32 [heads] or None joins the
+        denominator as exp(sinks[head])), zero behind it, into `rounded` and `rest` (bfloat16, same shape): the rounded weight and
+        what the rounding left."""
+        rows, keys = scores.shape
+        self._require(scores, "causal_softmax scores", torch.float32)
+        self._require(rounded, "causal_softmax rounded", torch.bfloat16, (rows, keys), scores)
+        self._require(rest, "causal_softmax rest", torch.bfloat16, (rows, keys), scores)
+        if sinks is not None:
+            self._require(sinks, "causal_softmax sinks", torch.float32, (heads,), scores)
+        self._check(self.lib.xrt_causal_softmax(_ptr(scores), ctypes.c_long(rows), ctypes.c_long(keys), int(heads), int(first_position),
+                                                ctypes.c_float(scale), _ptr(sinks), _ptr(rounded), _ptr(rest), self._stream(scores)))
+
+    def transpose(self, src, out):
+        """out[c, r] = src[r, c]; the rows of src may be columns of a wider matrix."""
+        rows, cols = src.shape
+        stride = self._rows(src, "transpose src")
+        self._require(out, "transpose out", src.dtype, (cols, rows), src)
+        self._check(self.lib.xrt_transpose(_ptr(src), ctypes.c_long(stride), _code(src), ctypes.c_long(rows), cols, _ptr(out), self._stream(src)))
 
     def latent_queries(self, q, heads, dim, rot_dim, frequencies, rot_dims, batch, plain, full, rank):
         """From the float32 rows q of heads x [plain (dim) | part to turn (rot_dim)]: the plain parts to `plain` [tokens, heads * dim],
@@ -1093,17 +1124,25 @@ class HipOps:
                                               self._stream(a)))
 
     # -- experts that multiply only the tokens that chose them
-    def _expert_matrices(self, w_gate_up, w_down, experts, width):
+    def _expert_matrices(self, w_gate_up, w_down, experts, width, stacked=False):
         """(data, packing, elements between two experts' matrices, row distance) of the gate/up matrix and of the down matrix, as
         `xrt_linear_groups` wants them, or None: [all gates | all ups] packed for a gated epilogue lies expert after expert
         already (a group of sixteen packed rows holds eight outputs' gate and up rows); an expert's down matrix is `width`
-        columns of the wide one."""
-        if not isinstance(w_gate_up, PackedMatrix) or w_gate_up.packing.kind != PACK_GATED or width % 64 != 0:
+        columns of the wide one. stacked: the gate/up matrix is a plain one that holds every expert's [gate rows | up rows] one
+        below the other (for experts whose activation reads float32 sums of both)."""
+        if width % 64 != 0:
             return None
         hidden = w_gate_up.shape[1]
-        if w_gate_up.packing.gated_n != experts * width or tuple(w_down.shape) != (hidden, experts * width):
-            return None
-        up = (w_gate_up.data, _Packing(PACK_GATED, width, 0, 0), 2 * width * hidden, hidden)
+        if stacked:
+            if isinstance(w_gate_up, PackedMatrix) or tuple(w_gate_up.shape) != (2 * experts * width, hidden) or tuple(w_down.shape) != (hidden, experts * width):
+                return None
+            up = (w_gate_up, None, 2 * width * hidden, hidden)
+        else:
+            if not isinstance(w_gate_up, PackedMatrix) or w_gate_up.packing.kind != PACK_GATED:
+                return None
+            if w_gate_up.packing.gated_n != experts * width or tuple(w_down.shape) != (hidden, experts * width):
+                return None
+            up = (w_gate_up.data, _Packing(PACK_GATED, width, 0, 0), 2 * width * hidden, hidden)
         if isinstance(w_down, PackedMatrix):
             if w_down.packing.kind != PACK_TILES:
                 return None
@@ -1112,10 +1151,10 @@ class HipOps:
             down = (w_down, None, width, experts * width)
         return up, down
 
-    def experts_sorted_takes(self, h, w_gate_up, w_down, experts, width, top) -> bool:
+    def experts_sorted_takes(self, h, w_gate_up, w_down, experts, width, top, stacked=False) -> bool:
         """Whether `experts_sorted` serves these operands, and pays: it multiplies every pick once, in tiles that are filled up
-        per expert, where the plain way multiplies every token with every expert."""
-        matrices = self._expert_matrices(w_gate_up, w_down, experts, width)
+        per expert, where the plain way multiplies every token with every expert. stacked: see `_expert_matrices`."""
+        matrices = self._expert_matrices(w_gate_up, w_down, experts, width, stacked)
         if matrices is None or h.dtype != torch.bfloat16 or h.dim() != 2 or h.shape[1] % 64 != 0 or experts > 256:
             return False
         tokens, hidden = h.shape
@@ -1123,21 +1162,24 @@ class HipOps:
         if tokens < 64 or 4 * tokens * experts < 5 * room or room // 128 > 65535:
             return False
         (up, up_packing, _, up_rows), (down, down_packing, _, down_rows) = matrices
-        return bool(self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, width, hidden, 2, ctypes.byref(up_packing))
-                    and self.lib.xrt_linear_groups_accepts(_ptr(h), width, _ptr(down), down_rows, hidden, width, 0,
+        takes_up = (self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, 2 * width, hidden, 0, None) if stacked else
+                    self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, width, hidden, 2, ctypes.byref(up_packing)))
+        return bool(takes_up and self.lib.xrt_linear_groups_accepts(_ptr(h), width, _ptr(down), down_rows, hidden, width, 0,
                                                            None if down_packing is None else ctypes.byref(down_packing)))
 
     def group_tile(self, tokens: int, top: int, experts: int) -> int:
         """Rows of a tile of sorted picks for a step of that many tokens."""
         return int(self.lib.xrt_linear_groups_tile_rows(ctypes.c_long(tokens), int(top), int(experts)))
 
-    def experts_sorted(self, h, w_gate_up, w_down, weights, chosen, width, out, activation: str = "silu"):
+    def experts_sorted(self, h, w_gate_up, w_down, weights, chosen, width, out, activation: str = "silu", clamp=None):
         """out[t] (float32) = sum over the experts e that token t chose, in the order of `chosen`, of weights[t, e] *
         W_down_e (act(W_gate_e h_t) * (W_up_e h_t)): the picks are sorted by expert, every expert multiplies its own rows, and
-        the outputs go back to their tokens. A token's result does not depend on what else the step holds."""
+        the outputs go back to their tokens. A token's result does not depend on what else the step holds.
+        clamp = (limit, alpha): the experts are clamped ones (`glu_clamped`) whose gate and up rows lie stacked expert after
+        expert in a plain matrix; their product keeps float32 sums, and the clamps and the activation are a pass of their own."""
         tokens, hidden = h.shape
         experts, top = weights.shape[1], chosen.shape[1]
-        matrices = self._expert_matrices(w_gate_up, w_down, experts, width)
+        matrices = self._expert_matrices(w_gate_up, w_down, experts, width, stacked=clamp is not None)
         if matrices is None:
             raise KernelError("experts_sorted: the experts' matrices do not lie expert after expert")
         (up, up_packing, up_stride, up_rows), (down, down_packing, down_stride, down_rows) = matrices
@@ -1155,9 +1197,15 @@ class HipOps:
         gathered = self._empty((room, hidden), torch.bfloat16, h.device)
         self._check(self.lib.xrt_gather_rows(_ptr(h), ctypes.c_long(h_stride), _ptr(rows), ctypes.c_long(room), hidden, _ptr(gathered), stream))
         act = self._empty((room, width), torch.bfloat16, h.device)
-        self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows, ctypes.byref(up_packing),
-                                               _ptr(act), _code(act), tile, ctypes.c_long(room // tile), width, hidden,
-                                               2 | (ACTIVATIONS[activation] << 8), _ptr(tile_group), 1, stream))
+        if clamp is not None:
+            sums = self._empty((room, 2 * width), torch.float32, h.device)
+            self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows, None, _ptr(sums), _code(sums),
+                                                   tile, ctypes.c_long(room // tile), 2 * width, hidden, 0, _ptr(tile_group), 1, stream))
+            self.glu_clamped(sums, act, float(clamp[0]), float(clamp[1]))
+        else:
+            self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows, ctypes.byref(up_packing),
+                                                   _ptr(act), _code(act), tile, ctypes.c_long(room // tile), width, hidden,
+                                                   2 | (ACTIVATIONS[activation] << 8), _ptr(tile_group), 1, stream))
         # (few tiles: the sum over an expert's width in two halves, which the last kernel adds)
         parts = int(self.lib.xrt_linear_groups_parts(ctypes.c_long(room // tile), hidden, width, 0))
         sorted_out = self._empty((room * parts, hidden), torch.float32, h.device)

@@ -194,8 +194,9 @@ class ExpertsMLP(FeedForward):
         self.w_router = runtime.matrix(tensors[self.router_name])
         total = self.experts * self.intermediate
         if self.clamp is not None:
-            # every expert's [gate rows | up rows] one below the other: the float32 sums of a token and an expert are one stretch
-            self.w_gate_up = runtime.weight([tensors[name] for names in self.expert_names for name in names[:2]])
+            # every expert's [gate rows | up rows] one below the other: the float32 sums of a token and an expert are one stretch,
+            # and an expert's rows are a matrix of their own for the product of sorted picks (a plain matrix: that product reads it so)
+            self.w_gate_up = runtime.stacked([tensors[name] for names in self.expert_names for name in names[:2]])
         else:
             # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]; packed for a gated epilogue the
             # former lies expert after expert, which is what the product of sorted picks reads
@@ -219,11 +220,13 @@ class ExpertsMLP(FeedForward):
         rt = self.runtime
         # A step of many tokens of which each uses few of the experts: the picks sorted by expert, every expert multiplies the
         # tokens that chose it. (Where the kernels have no such product, or it would not pay, every token meets every expert.)
-        takes = getattr(rt.ops, "experts_sorted_takes", None) if self.clamp is None else None
-        if takes is not None and takes(h, self.w_gate_up, self.w_down, self.experts, self.intermediate, self.top):
+        takes = getattr(rt.ops, "experts_sorted_takes", None)
+        stacked = {} if self.clamp is None else {"stacked": True}
+        if takes is not None and takes(h, self.w_gate_up, self.w_down, self.experts, self.intermediate, self.top, **stacked):
             chosen = rt.empty((h.shape[0], self.top), torch.int32)
             weights = self._weights(h, chosen)
-            rt.ops.experts_sorted(h, self.w_gate_up, self.w_down, weights, chosen, self.intermediate, out, activation="silu")
+            rt.ops.experts_sorted(h, self.w_gate_up, self.w_down, weights, chosen, self.intermediate, out,
+                                  **({"activation": "silu"} if self.clamp is None else {"clamp": self.clamp}))
             return
         weights = self._weights(h)
         act = rt.empty((h.shape[0], self.experts * self.intermediate))

@@ -15,6 +15,13 @@ head's key matrix, transposed, and the score is an ordinary one against the cach
 latents, and the head's value matrix turns that sum into the head's output. Both are products with a matrix per head
 (`ops.linear_heads`); the attention itself is the general kernel with H query heads on one key/value head.
 Norms, angles, scores and the softmax are float32; the products run in the compute dtype with float32 sums.
+
+A bfloat16 step whose sequences all start (prompts of some length) does not go through the attention kernel: the step has the
+prompts' cached rows at hand, so the scores of a stretch of queries, all heads at once, are one matrix product with those
+rows (float32 sums), a kernel turns them into the softmax's weights (as two bfloat16 numbers each, the rounded weight and what
+the rounding left), and two products with the latents, tokens along the rows, sum them up: the library's matrix-core products
+instead of a kernel that takes a key a lane. A query's weights behind its own position are zeros that the products still
+multiply: twice the arithmetic of a causal kernel, and still a twentieth of the time.
 """
 from __future__ import annotations
 
@@ -65,16 +72,62 @@ class LatentAttention(Mixer):
         self.w_uv = runtime.matrix(tensors[p + "uv"]).view(heads, self.value_dim, self.kv_rank)
         self.sink = tensors[p + self.sink_name].to(device=runtime.device, dtype=torch.float32).contiguous()
 
+    DENSE_FROM = 64                     # prompts from this many tokens on have their scores as a matrix product
+    DENSE_SCORES = 32 * 1024 * 1024     # most scores of a stretch of queries (float32: 128 MiB, and as much again for the weights)
+
+    def _prompts_alone(self, h, batch, cache) -> bool:
+        """Whether the step is one of prompts that start their sequences, long enough for the products of `_attend_prompts`."""
+        counts, starts = getattr(batch, "host_counts", None), getattr(batch, "host_starts", None)
+        if h.dtype != torch.bfloat16 or not cache.writable or not counts or starts is None or not hasattr(self.runtime.ops, "causal_softmax"):
+            return False
+        if sum(counts) != h.shape[0] or any(slot < 0 for slot in batch.host_slots):
+            return False
+        return all(start == 0 for start in starts) and min(counts) >= self.DENSE_FROM
+
+    def _attend_prompts(self, full, rows, batch, summed) -> None:
+        """summed[t, h] = the latents under the softmax's weights of query (t, h), for prompts that start their sequences:
+        full [tokens, heads * (rank + rot)] the queries, rows [tokens, rank + rot] the cached rows of the same tokens."""
+        rt = self.runtime
+        ops = rt.ops
+        heads, rank, width = self.n_heads, self.kv_rank, self.kv_rank + self.rot_dim
+        stretch_of = lambda count: max(1, min(count, self.DENSE_SCORES // (heads * count)))
+        # one set of buffers for all stretches of all prompts of the step, as large as the largest stretch needs
+        most = max(stretch_of(count) * heads * count for count in batch.host_counts)
+        most_sums = max(stretch_of(count) for count in batch.host_counts) * heads * rank
+        scores_all, sums_all = rt.empty((most,), torch.float32), rt.empty((most_sums,), torch.float32)
+        rounded_all, rest_all = rt.empty((most,)), rt.empty((most,))
+        latents_all = rt.empty((rank * max(batch.host_counts),))
+        at = 0
+        for count in batch.host_counts:
+            keys = rows[at:at + count]
+            latents = latents_all[:rank * count].view(rank, count)
+            ops.transpose(keys[:, :rank], latents)
+            stretch = stretch_of(count)
+            for first in range(0, count, stretch):
+                n = min(stretch, count - first)
+                shape = (n * heads, count)
+                queries = full[at + first:at + first + n].view(n * heads, width)
+                scores, rounded, rest = (flat[:n * heads * count].view(shape) for flat in (scores_all, rounded_all, rest_all))
+                ops.linear(queries, keys, scores)
+                ops.causal_softmax(scores, heads, first, self.scale, self.sink, rounded, rest)
+                sums = sums_all[:n * heads * rank].view(n * heads, rank)
+                ops.linear(rounded, latents, sums)
+                ops.linear(rest, latents, sums, accumulate=True)
+                ops.cast(sums, summed[at + first:at + first + n].view(n * heads, rank))
+            at += count
+
     def _heads_out(self, h, batch, cache):
         """The heads' outputs [tokens, n_heads * value_dim]."""
         rt = self.runtime
         ops = rt.ops
         tokens, heads, rank, rot = h.shape[0], self.n_heads, self.kv_rank, self.rot_dim
         frequencies = None if self.position is None else self.position.pair_rotation()[0]
+        prompts = self._prompts_alone(h, batch, cache)
+        rows = rt.empty((tokens, rank + rot)) if prompts else None
         if cache.writable:
             down = rt.empty((tokens, rank + rot), torch.float32)
             ops.linear(h, self.w_dkv, down)
-            ops.latent_complete(down, rank, rot, self.kv_gain, self.eps, frequencies, self.rot_dims, cache.kv, batch, like=h)
+            ops.latent_complete(down, rank, rot, self.kv_gain, self.eps, frequencies, self.rot_dims, cache.kv, batch, like=h, rows_out=rows)
         low = rt.empty((tokens, self.q_rank), torch.float32)
         ops.linear(h, self.w_dq, low)
         c_q = rt.empty((tokens, self.q_rank))
@@ -86,8 +139,11 @@ class LatentAttention(Mixer):
         ops.latent_queries(q, heads, self.dim, rot, frequencies, self.rot_dims, batch, plain, full, rank)
         ops.linear_heads(plain, self.w_uk_t, full, out_head=rank + rot)
         summed = rt.empty((tokens, heads * rank))
-        ops.attention(full, heads, 1, rank + rot, cache.kv, batch, summed, scale=self.scale, value_dim=rank, sink=self.sink,
-                      queries_alone=True)
+        if prompts:
+            self._attend_prompts(full, rows, batch, summed)
+        else:
+            ops.attention(full, heads, 1, rank + rot, cache.kv, batch, summed, scale=self.scale, value_dim=rank, sink=self.sink,
+                          queries_alone=True)
         out = rt.empty((tokens, heads * self.value_dim))
         ops.linear_heads(summed, self.w_uv, out)
         return out
