@@ -6,8 +6,9 @@ a matrix state per head with a fixed decay; `attention`, grouped softmax attenti
 sink, whose keys and values may be another layer's (`kv_from`); `latent_attention`, attention whose keys and values are
 made from a cached latent), the mixer's sizes under `mixer`, and `mlp`: a mixture of experts (`kind` "moe": `expert.ff`,
 `expert.limit`, `router.experts|top|scale|groups.count|groups.keep`) or null. Beside the layers: `vocab`, `width`,
-`norm.eps`, `streams` (the copies of the residual stream; absent: one plain residual stream without the copies' weights). The rows of an attention layer's table of biases are the
-table's first dimension; config.json may name them (`bias_rows`) or leave them to the checkpoint.
+`norm.eps`, `streams` (the copies of the residual stream; absent: one plain residual stream without the copies' weights).
+The rows of an attention layer's table of biases are the table's first dimension; config.json may name them (`bias_rows`)
+or leave them to the checkpoint.
 """
 from __future__ import annotations
 

@@ -310,8 +310,13 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
     // (what a lane then owns of a head fits two registers a head), where that still leaves two workgroups to a compute
     // unit (a decode step of few sequences would rather have the workgroups). Either way a head's arithmetic is the same.
     const int group = n_heads / n_kv_heads;
-    int together = max(head_dim, value_dim) > 2 * XRT_WAVE ? 1 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    // Heads larger than that take two together where the group is even: a key of some hundred dims is a long row of loads,
+    // which then serve both (the lanes' registers hold up to eight dims a head either way). (Tried also for steps of few
+    // tokens, a decode step of 8 sequences with 16 heads of 448 dims on one key/value head: 125 -> 164 us, the workgroups being half as many.)
+    const bool large = max(head_dim, value_dim) > 2 * XRT_WAVE;
+    int together = large ? (group % 2 == 0 ? 2 : 1) : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
     if ((long)tokens * (n_heads / together) < 2L * XRT_COMPUTE_UNITS) together = 1;
+    if (large && (size_t)2 * CHUNK_WAVES * together * value_dim * sizeof(float) > 48 * 1024) together = 1;      // (what the wavefronts' merge needs of LDS)
     const long items = (long)tokens * (n_heads / together);
     XRT_REQUIRE((long)tokens * n_heads < (1L << 31), "attention: too many (token, head) pairs");
     // rows of q, k and v side by side unless the caller says how far the rows of q lie apart
@@ -332,6 +337,7 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
 #define XRT_GENERIC_SETS(T)                                                                                               \
     do {                                                                                                                  \
         if (together == 4) XRT_GENERIC_WAVES(T, 4, 2);                                                                    \
+        else if (together == 2 && large) XRT_GENERIC_WAVES(T, 2, MAX_OWNED);                                              \
         else if (together == 2) XRT_GENERIC_WAVES(T, 2, 2);                                                               \
         else XRT_GENERIC_WAVES(T, 1, MAX_OWNED);                                                                          \
     } while (0)

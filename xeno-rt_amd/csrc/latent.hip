@@ -8,7 +8,8 @@
 //                        position * frequencies[i]; both into the cache
 //   xrt_latent_queries   from the queries' float32 sums, head by head [plain | part to turn]: the plain parts to rows of
 //                        their own, the turned parts to the tail of the rows that the attention kernel reads
-//   xrt_linear_heads     out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k], float32 sums in the order of k
+//   xrt_linear_heads     out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k], float32 sums (in the order of k for steps of many
+//                        rows, the lanes of a wavefront along k for steps of few)
 // A prompt that starts a sequence can have its scores as a matrix product of its own rows (all heads' queries of a stretch of
 // tokens against the prompt's cached rows, which the step has at hand): then
 //   xrt_causal_softmax   turns the float32 scores [queries x heads][keys] into the softmax's weights over the keys at or before
@@ -172,47 +173,58 @@ __global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ sr
         if (c0 + i < cols && r0 + tx < rows) dst[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
 }
 
-// The same product for a step of few rows (a decode step): a lane an output, the rows of a in LDS, the lane's row of w read
-// sixteen bytes at a time; every output's sum runs over k in the same order as in the tiles above, to the same bits.
-constexpr int HEADS_FEW = 16;
+// The same product for a step of few rows (a decode step): a wavefront an output column of one head, its lanes along k (a lane
+// takes sixteen bytes of the column's row of w at a time, and the same stretch of every row of a), the lanes' sums added in
+// the fixed order of the wavefront's butterfly. A row's result does not depend on the rows around it.
+constexpr int HEADS_FEW = 16, FEW_WAVES = 4;
 
 template <typename T>
-__global__ void __launch_bounds__(XRT_WAVE) linear_heads_few_kernel(const T* __restrict__ a, long a_stride, long a_head, const T* __restrict__ w,
-                                                                   T* __restrict__ out, long out_stride, long out_head, int rows, int n, int k) {
-    extern __shared__ float rows_of_a[];                       // [rows][k]
-    const int head = blockIdx.y, lane = threadIdx.x, column = blockIdx.x * XRT_WAVE + lane;
-    for (int e = lane; e < rows * k; e += XRT_WAVE) rows_of_a[e] = to_float(a[(long)(e / k) * a_stride + (long)head * a_head + e % k]);
-    wave_sync();
-    if (column >= n) return;
-    const T* mine = w + ((long)head * n + column) * k;
+__global__ void __launch_bounds__(FEW_WAVES * XRT_WAVE) linear_heads_few_kernel(const T* __restrict__ a, long a_stride, long a_head,
+                                                                               const T* __restrict__ w, T* __restrict__ out, long out_stride,
+                                                                               long out_head, int rows, int n, int k) {
+    const int head = blockIdx.y, lane = threadIdx.x % XRT_WAVE, column = blockIdx.x * FEW_WAVES + threadIdx.x / XRT_WAVE;
+    if (column >= n) return;                                   // (the whole wavefront)
+    const T* of_w = w + ((long)head * n + column) * k;
+    const T* of_a = a + (long)head * a_head;
+    constexpr int PIECE = 16 / sizeof(T);
+    struct alignas(16) Piece { T e[PIECE]; };
+    const bool whole = k % PIECE == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)a % 16 == 0 && a_stride % PIECE == 0 && a_head % PIECE == 0;
     float acc[HEADS_FEW];
 #pragma unroll
     for (int r = 0; r < HEADS_FEW; ++r) acc[r] = 0.f;
-    constexpr int PIECE = 16 / sizeof(T);
-    const bool whole = k % PIECE == 0 && (uintptr_t)w % 16 == 0;
-    for (int k0 = 0; k0 < k; k0 += PIECE) {
+    for (int k0 = lane * PIECE; k0 < k; k0 += XRT_WAVE * PIECE) {
         float piece[PIECE];
         if (whole) {
-            struct alignas(16) Piece { T e[PIECE]; };
-            const Piece loaded = *reinterpret_cast<const Piece*>(mine + k0);
+            const Piece loaded = *reinterpret_cast<const Piece*>(of_w + k0);
 #pragma unroll
             for (int e = 0; e < PIECE; ++e) piece[e] = to_float(loaded.e[e]);
         } else {
 #pragma unroll
-            for (int e = 0; e < PIECE; ++e) piece[e] = k0 + e < k ? to_float(mine[k0 + e]) : 0.f;
+            for (int e = 0; e < PIECE; ++e) piece[e] = k0 + e < k ? to_float(of_w[k0 + e]) : 0.f;
         }
 #pragma unroll
-        for (int e = 0; e < PIECE; ++e) {
-            if (k0 + e < k) {
+        for (int r = 0; r < HEADS_FEW; ++r) {
+            if (r < rows) {
+                const T* of_row = of_a + (long)r * a_stride + k0;
+                if (whole) {
+                    const Piece loaded = *reinterpret_cast<const Piece*>(of_row);
 #pragma unroll
-                for (int r = 0; r < HEADS_FEW; ++r)
-                    if (r < rows) acc[r] = fmaf(rows_of_a[r * k + k0 + e], piece[e], acc[r]);
+                    for (int e = 0; e < PIECE; ++e) acc[r] = fmaf(to_float(loaded.e[e]), piece[e], acc[r]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < PIECE; ++e)
+                        if (k0 + e < k) acc[r] = fmaf(to_float(of_row[e]), piece[e], acc[r]);
+                }
             }
         }
     }
 #pragma unroll
-    for (int r = 0; r < HEADS_FEW; ++r)
-        if (r < rows) out[(long)r * out_stride + (long)head * out_head + column] = from_float<T>(acc[r]);
+    for (int r = 0; r < HEADS_FEW; ++r) {
+        if (r < rows) {
+            const float sum = wave_sum(acc[r]);
+            if (lane == 0) out[(long)r * out_stride + (long)head * out_head + column] = from_float<T>(sum);
+        }
+    }
 }
 
 }  // namespace
@@ -289,15 +301,14 @@ extern "C" int xrt_linear_heads(const void* a, long a_stride, long a_head, const
     XRT_REQUIRE(a_head >= k && a_stride >= (heads - 1) * a_head + k && out_head >= n && out_stride >= (heads - 1) * out_head + n,
                 "linear_heads: rows %ld and %ld apart do not hold %d heads %ld and %ld apart", a_stride, out_stride, heads, a_head, out_head);
     if (rows == 0) return 0;
-    if (rows <= HEADS_FEW && (size_t)rows * k * sizeof(float) <= 48 * 1024) {
-        const dim3 few((n + XRT_WAVE - 1) / XRT_WAVE, heads);
-        const size_t lds = (size_t)rows * k * sizeof(float);
+    if (rows <= HEADS_FEW) {
+        const dim3 few((n + FEW_WAVES - 1) / FEW_WAVES, heads);
         if (dtype == XRT_F32)
-            linear_heads_few_kernel<float><<<few, XRT_WAVE, lds, (hipStream_t)stream>>>((const float*)a, a_stride, a_head, (const float*)w, (float*)out,
-                                                                                      out_stride, out_head, (int)rows, n, k);
+            linear_heads_few_kernel<float><<<few, FEW_WAVES * XRT_WAVE, 0, (hipStream_t)stream>>>((const float*)a, a_stride, a_head, (const float*)w,
+                                                                                               (float*)out, out_stride, out_head, (int)rows, n, k);
         else
-            linear_heads_few_kernel<bf16><<<few, XRT_WAVE, lds, (hipStream_t)stream>>>((const bf16*)a, a_stride, a_head, (const bf16*)w, (bf16*)out,
-                                                                                     out_stride, out_head, (int)rows, n, k);
+            linear_heads_few_kernel<bf16><<<few, FEW_WAVES * XRT_WAVE, 0, (hipStream_t)stream>>>((const bf16*)a, a_stride, a_head, (const bf16*)w,
+                                                                                              (bf16*)out, out_stride, out_head, (int)rows, n, k);
         XRT_LAUNCH_CHECK("linear_heads");
         return 0;
     }
