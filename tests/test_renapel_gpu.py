@@ -433,6 +433,33 @@ def test_one_key_far_back_or_at_a_blocks_border_is_found(key, ops):
         assert abs(float(got[-1, 0]) - 7.0) < 2e-2 and abs(float(got[-1, vdim]) - 7.0) < 2e-2, f"key {key}, cuts {cuts[:2]}"
 
 
+@pytest.mark.parametrize("n_heads,dim,vdim", [(16, 128, 96), (6, 128, 96), (20, 64, 32), (5, 448, 384), (33, 96, 64), (1, 32, 32)])
+def test_many_heads_on_one_key_value_head_on_the_matrix_cores(n_heads, dim, vdim, ops):
+    """bfloat16, one key/value head, key and value sizes in whole tiles: the kernel that takes sixteen heads of a token as the
+    columns of its score tiles, against plain arithmetic, for every way to cut the sequence; then one key far back or at a
+    block's border whose score towers over the others."""
+    length = 150
+    generator = torch.Generator().manual_seed(dim + vdim + n_heads)
+    q, k, v = (torch.randn(length, width, generator=generator).bfloat16().float() for width in (n_heads * dim, dim, vdim))
+    sink = 2.0 * torch.randn(n_heads, generator=generator)
+    scale = 0.6 / math.sqrt(dim)
+    want = plain_attention_with_sink(q, k, v, n_heads, 1, dim, vdim, scale, sink)
+    for cuts in schedules(length):
+        got = attend(ops, q, k, v, cuts, torch.bfloat16, n_heads, 1, dim, vdim, scale=scale, sink=sink.cuda())
+        assert float((got - want).abs().max()) <= 2e-2 * float(want.abs().max()), f"cuts {cuts[:4]}"
+    want = plain_attention_with_sink(q, k, v, n_heads, 1, dim, vdim, scale, torch.full((n_heads,), -math.inf))
+    got = attend(ops, q, k, v, [length - 9] + [1] * 9, torch.bfloat16, n_heads, 1, dim, vdim, scale=scale)
+    assert float((got - want).abs().max()) <= 2e-2 * float(want.abs().max()), "without a sink"
+    length = 900
+    for key in (0, 1, 63, 64, 65, 511, 512, 700):
+        q, k, v = (0.1 * torch.randn(length, width, generator=generator) for width in (n_heads * dim, dim, vdim))
+        q[-1], k[key] = 3.0, 3.0
+        v[key] = 7.0
+        for cuts in ([length - 33] + [1] * 33, [key + 1, length - key - 2, 1]):
+            got = attend(ops, q, k, v, cuts, torch.bfloat16, n_heads, 1, dim, vdim, scale=0.1 * 32 / dim, sink=sink.cuda())
+            assert abs(float(got[-1, 0]) - 7.0) < 5e-2 and abs(float(got[-1, -1]) - 7.0) < 5e-2, f"key {key}, cuts {cuts[:2]}"
+
+
 def test_queries_are_completed_with_plain_norms_and_a_temperature(ops):
     """What lies between the projection and the scores: biases, every head divided by its root mean square, and the queries
     times a temperature that steps up with the position, in prompts and decoded, also for a layer that projects queries only."""
@@ -499,7 +526,8 @@ def run_step(part, h, at, cache, dtype):
 @pytest.mark.parametrize("m", [dict(heads=3, dim=16, rot_dim=8, vdim=12, kv_rank=24, q_rank=20, scale=0.2, rot={"dims": 8, "base": 1000.0}),
                                dict(heads=1, dim=40, rot_dim=16, vdim=72, kv_rank=80, q_rank=12, scale=0.15, rot={"dims": 8, "base": 10000.0}),
                                dict(heads=5, dim=8, rot_dim=6, vdim=4, kv_rank=40, q_rank=48, scale=0.3, rot={"dims": 2, "base": 10.0}),
-                               dict(heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=160, q_rank=96, scale=0.1, rot={"dims": 32, "base": 250.0})])
+                               dict(heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=160, q_rank=96, scale=0.1, rot={"dims": 32, "base": 250.0}),
+                               dict(heads=18, dim=24, rot_dim=32, vdim=16, kv_rank=96, q_rank=40, scale=0.2, rot={"dims": 16, "base": 5000.0})])
 def test_latent_attention_alone(m, dtype, ops):
     from xeno_rt_amd.models.renapel import _mixer
     width, length = 48, 150

@@ -463,6 +463,18 @@ int xrt_latent_queries(const float* q, long q_stride, int dtype, long tokens, in
 int xrt_linear_heads(const void* a, long a_stride, long a_head, const void* w, int dtype, void* out, long out_stride, long out_head,
                      long rows, int heads, int n, int k, void* stream);
 
+// ---- many heads on one key/value head with large keys, on the matrix cores (csrc/attention_latent.hip) ------------------------
+// Causal attention of the step's tokens (queries alone in q, rows q_stride apart, n_heads x head_dim each) over a cache with one
+// key/value head, keys of head_dim and values of value_dim numbers (multiples of 32 up to 512: `accepts`), bfloat16; with
+// sink_scores (float32 [n_heads], or null) the softmax's denominator also holds exp(sink_scores[head]). out: rows of
+// n_heads x value_dim. max_context: the longest sequence after this step; the workspace holds `xrt_attention_latent_workspace` floats.
+int xrt_attention_latent_accepts(int dtype, int n_kv_heads, int head_dim, int value_dim);
+long xrt_attention_latent_workspace(long tokens, int n_heads, int value_dim, int max_context);
+int xrt_attention_latent(const void* q, long q_stride, long tokens, int n_heads, int head_dim, int value_dim, const void* k_cache,
+                         const void* v_cache, const int* block_table, int table_stride, int n_blocks, const int* positions,
+                         const int* slots, void* out, float scale, const float* sink_scores, int max_context, float* workspace,
+                         long workspace_floats, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

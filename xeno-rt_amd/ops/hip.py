@@ -202,7 +202,8 @@ class HipOps:
                      "xrt_route_experts", "xrt_scale_blocks", "xrt_attention_stretches", "xrt_attention_stretches_accepts",
                      "xrt_experts_sort", "xrt_gather_rows", "xrt_linear_groups", "xrt_linear_groups_accepts", "xrt_experts_combine",
                      "xrt_linear_groups_tile_rows", "xrt_linear_groups_parts", "xrt_streams_open", "xrt_streams_read", "xrt_streams_write",
-                     "xrt_latent_complete", "xrt_latent_queries", "xrt_linear_heads", "xrt_causal_softmax", "xrt_transpose"):
+                     "xrt_latent_complete", "xrt_latent_queries", "xrt_linear_heads", "xrt_causal_softmax", "xrt_transpose", "xrt_attention_latent",
+                     "xrt_attention_latent_accepts"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -217,6 +218,7 @@ class HipOps:
         self.lib.xrt_attention_sigmoid_workspace.restype = ctypes.c_long
         self.lib.xrt_selective_scan_workspace.restype = ctypes.c_long
         self.lib.xrt_experts_sort_room.restype = ctypes.c_long
+        self.lib.xrt_attention_latent_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -504,6 +506,10 @@ class HipOps:
                 and self._attention_stretches(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, chunk,
                                               distance_bias, sink if isinstance(sink, torch.Tensor) else None)):
             return None
+        if (queries_alone and n_kv_heads == 1 and sink is not True and distance_bias is None and distance_slopes is None and not window and not chunk
+                and self._attention_one_kv_head(qkv, n_heads, head_dim, value_dim or head_dim, kv, batch, out, scale,
+                                                sink if isinstance(sink, torch.Tensor) else None)):
+            return None
         if sink is not False or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone or chunk:
             return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
                                            distance_slopes, sink, distance_bias, queries_alone, chunk)
@@ -539,6 +545,30 @@ class HipOps:
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
             ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
+
+    def _attention_one_kv_head(self, q, n_heads, head_dim, value_dim, kv, batch, out, scale, sink_scores) -> bool:
+        """The matrix-core kernel for many query heads on one key/value head (the queries alone in `q`; bfloat16, key and value
+        sizes that are multiples of 32 up to 512). False: not served here, and nothing was done."""
+        tokens = q.shape[0]
+        max_context = int(getattr(batch, "max_context", 0) or 0)
+        if tokens > 65535 or max_context <= 0 or not self.lib.xrt_attention_latent_accepts(_code(q), 1, head_dim, value_dim):
+            return False
+        q_stride = self._rows(q, "attention q", n_heads * head_dim)
+        if q_stride % 8 != 0 or q.data_ptr() % 16 != 0:
+            return False
+        self._require(out, "attention out", q.dtype, (tokens, n_heads * value_dim), q)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), q)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), q)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, q, 1, head_dim, value_dim)
+        if sink_scores is not None:
+            self._require(sink_scores, "attention sink", torch.float32, (n_heads,), q)
+        need = int(self.lib.xrt_attention_latent_workspace(ctypes.c_long(tokens), n_heads, value_dim, max_context))
+        workspace = self._empty(need, torch.float32, q.device)
+        self._check(self.lib.xrt_attention_latent(
+            _ptr(q), ctypes.c_long(q_stride), ctypes.c_long(tokens), n_heads, head_dim, value_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table), stride,
+            n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale), _ptr(sink_scores), max_context, _ptr(workspace),
+            ctypes.c_long(need), self._stream(q)))
+        return True
 
     def _attention_stretches(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, chunk, distance_bias=None,
                              sink_scores=None) -> bool:
