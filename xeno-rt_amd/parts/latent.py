@@ -13,7 +13,9 @@ What is cached per token is one row [c | turned key part] as the key of a single
 per-head keys never exist: q_plain . (W_uk,h c) = (W_uk,h^T q_plain) . c, so the plain part of a query is multiplied by its
 head's key matrix, transposed, and the score is an ordinary one against the cached row; the softmax's weights sum the
 latents, and the head's value matrix turns that sum into the head's output. Both are products with a matrix per head
-(`ops.linear_heads`); the attention itself is the general kernel with H query heads on one key/value head.
+(`ops.linear_heads`); the attention itself is `ops.attention` with H query heads on one key/value head, which in bfloat16
+takes the matrix-core kernel for such a cache (sixteen heads of a token as the columns of a score tile) where the key and
+value sizes are whole tiles of 32, and the general kernel otherwise.
 Norms, angles, scores and the softmax are float32; the products run in the compute dtype with float32 sums.
 
 A bfloat16 step whose sequences all start (prompts of some length) does not go through the attention kernel: the step has the
