@@ -562,7 +562,8 @@ def test_latent_attention_alone(m, dtype, ops):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("tokens,heads,n,k", [(1, 3, 24, 16), (70, 5, 40, 8), (200, 1, 80, 72), (65, 8, 160, 64), (9, 2, 3, 130)])
+@pytest.mark.parametrize("tokens,heads,n,k", [(1, 3, 24, 16), (70, 5, 40, 8), (200, 1, 80, 72), (65, 8, 160, 64), (9, 2, 3, 130), (300, 16, 384, 128),
+                                              (100, 4, 96, 96), (17, 3, 50, 32)])
 def test_products_with_a_matrix_per_head(tokens, heads, n, k, dtype, ops):
     generator = torch.Generator().manual_seed(n + k)
     a, w = torch.randn(tokens, heads * k, generator=generator).to(dtype), torch.randn(heads, n, k, generator=generator).to(dtype)

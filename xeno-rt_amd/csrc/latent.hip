@@ -8,8 +8,8 @@
 //                        position * frequencies[i]; both into the cache
 //   xrt_latent_queries   from the queries' float32 sums, head by head [plain | part to turn]: the plain parts to rows of
 //                        their own, the turned parts to the tail of the rows that the attention kernel reads
-//   xrt_linear_heads     out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k], float32 sums (in the order of k for steps of many
-//                        rows, the lanes of a wavefront along k for steps of few)
+//   xrt_linear_heads     out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k], float32 sums (steps of many rows: on the matrix cores in
+//                        bfloat16 with k in whole steps of 32, else in the order of k; steps of few: the lanes of a wavefront along k)
 // A prompt that starts a sequence can have its scores as a matrix product of its own rows (all heads' queries of a stretch of
 // tokens against the prompt's cached rows, which the step has at hand): then
 //   xrt_causal_softmax   turns the float32 scores [queries x heads][keys] into the softmax's weights over the keys at or before
@@ -173,6 +173,45 @@ __global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ sr
         if (c0 + i < cols && r0 + tx < rows) dst[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
 }
 
+// The same product on the matrix cores, for bfloat16 steps of many rows with k in whole steps of 32: a wavefront takes 16 rows
+// and 64 outputs of one head; both operands of v_mfma_f32_16x16x32_bf16 come straight from memory, sixteen bytes a lane (a row
+// of a: 8 consecutive k of one token; a row of w: 8 consecutive k of one output), nothing passes LDS.
+typedef __bf16 heads_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float heads_floatx4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256) linear_heads_mfma_kernel(const bf16* __restrict__ a, long a_stride, long a_head, const bf16* __restrict__ w,
+                                                               bf16* __restrict__ out, long out_stride, long out_head, long rows, int n, int k) {
+    const int head = blockIdx.z, lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE, r = lane % 16, c = lane / 16;
+    const long row0 = (long)blockIdx.x * 64 + wave * 16;
+    if (row0 >= rows) return;                                  // (the whole wavefront)
+    const int n0 = blockIdx.y * 64;
+    const bf16* of_a = a + min(row0 + r, rows - 1) * a_stride + (long)head * a_head + c * 8;
+    const bf16* of_w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) of_w[j] = w + ((long)head * n + min(n0 + 16 * j + r, n - 1)) * k + c * 8;
+    heads_floatx4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = heads_floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+    for (int k0 = 0; k0 < k; k0 += 32) {
+        const heads_bf16x8 of_rows = *reinterpret_cast<const heads_bf16x8*>(of_a + k0);
+        heads_bf16x8 of_outputs[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) of_outputs[j] = *reinterpret_cast<const heads_bf16x8*>(of_w[j] + k0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(of_rows, of_outputs[j], acc[j], 0, 0, 0);
+    }
+    // register i of tile j is row row0 + 4 c + i, output n0 + 16 j + r
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const long row = row0 + 4 * c + i;
+            const int column = n0 + 16 * j + r;
+            if (row < rows && column < n) out[row * out_stride + (long)head * out_head + column] = (bf16)acc[j][i];
+        }
+}
+
 // The same product for a step of few rows (a decode step): a wavefront an output column of one head, its lanes along k (a lane
 // takes sixteen bytes of the column's row of w at a time, and the same stretch of every row of a), the lanes' sums added in
 // the fixed order of the wavefront's butterfly. A row's result does not depend on the rows around it.
@@ -309,6 +348,14 @@ extern "C" int xrt_linear_heads(const void* a, long a_stride, long a_head, const
         else
             linear_heads_few_kernel<bf16><<<few, FEW_WAVES * XRT_WAVE, 0, (hipStream_t)stream>>>((const bf16*)a, a_stride, a_head, (const bf16*)w,
                                                                                               (bf16*)out, out_stride, out_head, (int)rows, n, k);
+        XRT_LAUNCH_CHECK("linear_heads");
+        return 0;
+    }
+    if (dtype == XRT_BF16 && k % 32 == 0 && a_stride % 8 == 0 && a_head % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+        (rows + 63) / 64 < (1L << 31) && (n + 63) / 64 <= 65535) {
+        const dim3 tiles((unsigned)((rows + 63) / 64), (n + 63) / 64, heads);
+        linear_heads_mfma_kernel<<<tiles, 256, 0, (hipStream_t)stream>>>((const bf16*)a, a_stride, a_head, (const bf16*)w, (bf16*)out, out_stride, out_head,
+                                                                         rows, n, k);
         XRT_LAUNCH_CHECK("linear_heads");
         return 0;
     }

@@ -447,7 +447,8 @@ int xrt_streams_write(float* streams, int copies, const float* mix, const float*
 // queries: from float32 rows of heads x [plain (dim) | part to turn (rot_dim)] the plain parts to `plain` [tokens][heads][dim]
 // and the turned parts to full[t][h][rank ..], rows full_stride apart, heads rank + rot_dim apart.
 // linear_heads: out[t][h][n] = sum over k of a[t][h][k] * w[h][n][k]; rows of a and out a_stride and out_stride apart, heads
-// a_head and out_head apart; all three of `dtype`, float32 sums (whose order depends on whether the step has up to 16 rows or more, on nothing else).
+// a_head and out_head apart; all three of `dtype`, float32 sums (whose order depends on whether the step has up to 16 rows or more and on
+// the sizes, on nothing else: a row's result never depends on the rows around it).
 int xrt_latent_complete(const float* down, long down_stride, int dtype, long tokens, int rank, int rot_dim, int rot_dims,
                         const void* gain, int gain_dtype, float eps, const float* frequencies, const int* positions, const int* slots,
                         void* k_cache, void* v_cache, const int* block_table, int table_stride, int n_blocks, void* rows_out, void* stream);
