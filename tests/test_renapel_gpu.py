@@ -632,8 +632,9 @@ def test_clamped_experts_alone(mlp, dtype, ops):
     assert float((alone[0] - out[17]).abs().max()) <= 1e-5 * float(want.abs().max()) if dtype == torch.float32 else True
 
 
+@pytest.mark.parametrize("pack", ["auto", "always", False])
 @pytest.mark.parametrize("ff,experts,top,groups,tokens", [(64, 8, 2, (4, 2), 300), (128, 16, 4, None, 1000), (192, 4, 1, (2, 1), 600)])
-def test_clamped_experts_multiply_only_the_tokens_that_chose_them(ff, experts, top, groups, tokens, ops):
+def test_clamped_experts_multiply_only_the_tokens_that_chose_them(ff, experts, top, groups, tokens, pack, ops):
     """A step of many tokens sorts its picks by expert: against the plain sum, and against the same part with every token
     through every expert (the same choices, so rounding alone differs)."""
     from renapel_models import _moe
@@ -642,7 +643,9 @@ def test_clamped_experts_multiply_only_the_tokens_that_chose_them(ff, experts, t
     raw = _moe(ff, 1.5, experts, top, groups, 2.0)
     part = _feed_forward(raw, "mlp.", types.SimpleNamespace(width=width))
     tensors = tensors_for(part, seed=ff, std=0.3, router=(0.0, 0.7))
-    part.bind(tensors, runtime(ops, torch.bfloat16))
+    from xeno_rt_amd.parts.base import Runtime
+    part.bind(tensors, Runtime(ops, torch.bfloat16, "cuda", pack_weights=pack))       # (the stacked gate/up matrix plain, and in tiles)
+    assert pack != "always" or hasattr(part.w_gate_up, "unpacked")
     h = torch.randn(tokens, width, generator=torch.Generator().manual_seed(6)).bfloat16()
     assert ops.experts_sorted_takes(h.cuda(), part.w_gate_up, part.w_down, experts, ff, top, stacked=True)
     assert not ops.experts_sorted_takes(h[:8].cuda(), part.w_gate_up, part.w_down, experts, ff, top, stacked=True)

@@ -387,8 +387,10 @@ int xrt_gated_rows(const float* s, long s_stride, const void* table, int table_d
 // copy (or null): the updated rows once more, in copy_dtype
 int xrt_add_weighted(float* residual, int count, const float* const* y, const void* const* gains, const float* scales, int gain_dtype,
                      long rows, int width, void* copy, int copy_dtype, void* stream);
-// out[r][c] = g * sigmoid(alpha * g) * (u + 1), g = min(sums[r][c], limit), u = clamp(sums[r][n + c], -limit, limit)
-int xrt_glu_clamped(const float* sums, void* out, int out_dtype, long rows, int n, float limit, float alpha, void* stream);
+// out[r][c] = g * sigmoid(alpha * g) * (u + 1), g = min(sums[r][c], limit), u = clamp(sums[r][n + c], -limit, limit); times
+// row_weights[r] (float32 [rows]) unless that is null
+int xrt_glu_clamped(const float* sums, void* out, int out_dtype, long rows, int n, float limit, float alpha, const float* row_weights,
+                    void* stream);
 // x <- cap * tanh(x / cap), float32 in place
 int xrt_softcap(float* x, long count, float cap, void* stream);
 int xrt_cast(const void* x, int x_dtype, void* out, int out_dtype, long count, void* stream);

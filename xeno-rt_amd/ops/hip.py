@@ -1005,13 +1005,18 @@ class HipOps:
         self._check(self.lib.xrt_add_weighted(_ptr(residual), count, ys, gs, scales, _code(gains[0]) if gains else 0, ctypes.c_long(rows),
                                               width, _ptr(copy), 0 if copy is None else _code(copy), self._stream(residual)))
 
-    def glu_clamped(self, sums, out, limit, alpha):
-        """out = g * sigmoid(alpha g) * (u + 1) with g = min(sums[:, :n], limit), u = clamp(sums[:, n:], -limit, limit)."""
+    def glu_clamped(self, sums, out, limit, alpha, row_weights=None):
+        """out = g * sigmoid(alpha g) * (u + 1) with g = min(sums[:, :n], limit), u = clamp(sums[:, n:], -limit, limit); every row
+        times its entry of row_weights (float32, one number a row in any shape), if given."""
         rows, n = out.shape
         self._require(sums, "glu_clamped sums", torch.float32, (rows, 2 * n))
         self._require(out, "glu_clamped out", None, (rows, n), sums)
+        if row_weights is not None:
+            self._require(row_weights, "glu_clamped row_weights", torch.float32, None, sums)
+            if row_weights.numel() != rows:
+                raise KernelError(f"glu_clamped row_weights: {row_weights.numel()} numbers for {rows} rows")
         self._check(self.lib.xrt_glu_clamped(_ptr(sums), _ptr(out), _code(out), ctypes.c_long(rows), n, ctypes.c_float(limit),
-                                             ctypes.c_float(alpha), self._stream(sums)))
+                                             ctypes.c_float(alpha), _ptr(row_weights), self._stream(sums)))
 
     def softcap(self, x, cap):
         """x <- cap * tanh(x / cap), in place; x float32."""
@@ -1164,9 +1169,14 @@ class HipOps:
             return None
         hidden = w_gate_up.shape[1]
         if stacked:
-            if isinstance(w_gate_up, PackedMatrix) or tuple(w_gate_up.shape) != (2 * experts * width, hidden) or tuple(w_down.shape) != (hidden, experts * width):
+            if tuple(w_gate_up.shape) != (2 * experts * width, hidden) or tuple(w_down.shape) != (hidden, experts * width):
                 return None
-            up = (w_gate_up, None, 2 * width * hidden, hidden)
+            if isinstance(w_gate_up, PackedMatrix):            # in tiles of 16 rows, an expert's rows (a multiple of 128) begin where they would unpacked
+                if w_gate_up.packing.kind != PACK_TILES:
+                    return None
+                up = (w_gate_up.data, w_gate_up.packing, 2 * width * hidden, hidden)
+            else:
+                up = (w_gate_up, None, 2 * width * hidden, hidden)
         else:
             if not isinstance(w_gate_up, PackedMatrix) or w_gate_up.packing.kind != PACK_GATED:
                 return None
@@ -1192,7 +1202,8 @@ class HipOps:
         if tokens < 64 or 4 * tokens * experts < 5 * room or room // 128 > 65535:
             return False
         (up, up_packing, _, up_rows), (down, down_packing, _, down_rows) = matrices
-        takes_up = (self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, 2 * width, hidden, 0, None) if stacked else
+        takes_up = (self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, 2 * width, hidden, 0,
+                                                       None if up_packing is None else ctypes.byref(up_packing)) if stacked else
                     self.lib.xrt_linear_groups_accepts(_ptr(h), hidden, _ptr(up), up_rows, width, hidden, 2, ctypes.byref(up_packing)))
         return bool(takes_up and self.lib.xrt_linear_groups_accepts(_ptr(h), width, _ptr(down), down_rows, hidden, width, 0,
                                                            None if down_packing is None else ctypes.byref(down_packing)))
@@ -1229,7 +1240,8 @@ class HipOps:
         act = self._empty((room, width), torch.bfloat16, h.device)
         if clamp is not None:
             sums = self._empty((room, 2 * width), torch.float32, h.device)
-            self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows, None, _ptr(sums), _code(sums),
+            self._check(self.lib.xrt_linear_groups(_ptr(gathered), hidden, _ptr(up), ctypes.c_long(up_stride), up_rows,
+                                                   None if up_packing is None else ctypes.byref(up_packing), _ptr(sums), _code(sums),
                                                    tile, ctypes.c_long(room // tile), 2 * width, hidden, 0, _ptr(tile_group), 1, stream))
             self.glu_clamped(sums, act, float(clamp[0]), float(clamp[1]))
         else:

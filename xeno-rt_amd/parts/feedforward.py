@@ -195,8 +195,8 @@ class ExpertsMLP(FeedForward):
         total = self.experts * self.intermediate
         if self.clamp is not None:
             # every expert's [gate rows | up rows] one below the other: the float32 sums of a token and an expert are one stretch,
-            # and an expert's rows are a matrix of their own for the product of sorted picks (a plain matrix: that product reads it so)
-            self.w_gate_up = runtime.stacked([tensors[name] for names in self.expert_names for name in names[:2]])
+            # and an expert's rows are a matrix of their own for the product of sorted picks
+            self.w_gate_up = runtime.weight([tensors[name] for names in self.expert_names for name in names[:2]])
         else:
             # [all gates | all ups] x hidden, and hidden x [every expert's stretch of the activations]; packed for a gated epilogue the
             # former lies expert after expert, which is what the product of sorted picks reads
@@ -233,10 +233,11 @@ class ExpertsMLP(FeedForward):
         if self.clamp is not None:
             sums = rt.empty((h.shape[0], 2 * self.experts * self.intermediate), torch.float32)
             rt.ops.linear(h, self.w_gate_up, sums)
-            rt.ops.glu_clamped(sums.view(-1, 2 * self.intermediate), act.view(-1, self.intermediate), *self.clamp)
+            # (the router's weights ride along: a row of the sums is a (token, expert) pair)
+            rt.ops.glu_clamped(sums.view(-1, 2 * self.intermediate), act.view(-1, self.intermediate), *self.clamp, row_weights=weights)
         else:
             rt.ops.linear_glu(h, self.w_gate_up, act, activation="silu")
-        rt.ops.scale_blocks(act, weights, self.intermediate)
+            rt.ops.scale_blocks(act, weights, self.intermediate)
         rt.ops.linear(act, self.w_down, out)
 
     def forward(self, h, batch, residual: torch.Tensor) -> None:
